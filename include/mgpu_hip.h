@@ -1,0 +1,185 @@
+/*
+ * libmgpu_hip -- C ABI of the MI355X (gfx950) implementation of moderngpu's
+ * load-balancing-search / segmented-reduce path.
+ *
+ * The reference library is header-only C++ templates; it has no FFI of its
+ * own.  These entry points are what its public templates bind to for raw
+ * pointer arguments and the built-in operators, and what any other host
+ * language binds to directly.  Each declaration cites the reference template
+ * it stands for (paths relative to the moderngpu tree).
+ *
+ * Conventions
+ *  - All pointers are device pointers unless stated otherwise.
+ *  - All work is enqueued on `stream` (a hipStream_t passed as void*; NULL is
+ *    the default stream).  No entry point synchronises, allocates or frees;
+ *    temporaries live in the caller-provided workspace, whose required size
+ *    comes from the matching *_workspace_bytes function.  The workspace must
+ *    stay untouched until the enqueued work has completed.
+ *  - Return value: 0 (hipSuccess) or a hipError_t code.  Nothing throws.
+ *  - Index type is 32-bit int throughout, as in the reference:
+ *    count + num_segments must be < 2^31.
+ *  - segments[] holds the ascending start index of every segment,
+ *    segments[0] == 0, with no trailing `count` entry; equal consecutive
+ *    starts denote an empty segment.
+ */
+#ifndef MGPU_HIP_H
+#define MGPU_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MGPU_HIP_API __attribute__((visibility("default")))
+
+typedef void* mgpu_stream_t;
+
+/* Value types (operators.hxx:91-124 are templates over the value type). */
+enum {
+  MGPU_I32 = 0, MGPU_U32 = 1, MGPU_I64 = 2, MGPU_U64 = 3,
+  MGPU_F32 = 4, MGPU_F64 = 5
+};
+/* mgpu::plus_t, mgpu::maximum_t, mgpu::minimum_t (operators.hxx:91-124). */
+enum { MGPU_PLUS = 0, MGPU_MAXIMUM = 1, MGPU_MINIMUM = 2 };
+/* mgpu::bounds_lower / bounds_upper (types.hxx:81-84). */
+enum { MGPU_BOUNDS_LOWER = 0, MGPU_BOUNDS_UPPER = 1 };
+/* Phase masks for the *_phases entry points (measurement only). */
+enum { MGPU_PHASE_PARTITION = 1, MGPU_PHASE_TILES = 2, MGPU_PHASE_SPINE = 4,
+       MGPU_PHASE_ALL = 7 };
+
+/* Library version, major * 10000 + minor * 100 + patch. */
+MGPU_HIP_API int mgpu_hip_version(void);
+/* Text for a return code (hipGetErrorString). */
+MGPU_HIP_API const char* mgpu_hip_error_string(int code);
+/* Tile size nv = nt * vt (merged elements per CTA) the library uses for
+ * segreduce on `dtype`, and for the load-balancing search. */
+MGPU_HIP_API int mgpu_hip_segreduce_tile_size(int dtype);
+MGPU_HIP_API int mgpu_hip_lbs_tile_size(void);
+
+/* ---- partitioning ------------------------------------------------------ */
+
+/* Number of entries the partition functions write:
+ * div_up(a_count + b_count, spacing) + 1  (search.hxx:18). */
+MGPU_HIP_API int mgpu_hip_partition_count(int64_t a_count, int64_t b_count,
+  int64_t spacing);
+
+/* mgpu::load_balance_partitions (search.hxx:29-37): partitions[i] = merge
+ * path split of cross-diagonal min(spacing * i, count + num_segments) between
+ * the item indices [0, count) and the segment starts, bounds_upper. */
+MGPU_HIP_API int mgpu_hip_load_balance_partitions(int64_t count,
+  const int* segments, int num_segments, int spacing, int* partitions,
+  mgpu_stream_t stream);
+
+/* mgpu::merge_path_partitions<bounds> (search.hxx:12-27) for int keys with
+ * less_t.  a_keys == NULL means the counting sequence 0, 1, 2, ... */
+MGPU_HIP_API int mgpu_hip_merge_path_partitions(const int* a_keys,
+  int64_t a_count, const int* b_keys, int64_t b_count, int64_t spacing,
+  int bounds, int* partitions, mgpu_stream_t stream);
+
+/* mgpu::binary_search_partitions<bounds> (search.hxx:39-51). */
+MGPU_HIP_API int mgpu_hip_binary_search_partitions(const int* keys, int count,
+  int num_items, int spacing, int bounds, int* partitions,
+  mgpu_stream_t stream);
+
+/* ---- segmented reduction ----------------------------------------------- */
+
+/* Bytes of workspace mgpu_hip_segreduce / mgpu_hip_spmv need. */
+MGPU_HIP_API size_t mgpu_hip_segreduce_workspace_bytes(int count,
+  int num_segments, int dtype);
+
+/* mgpu::segreduce (kernel_segreduce.hxx:193-268) for pointer inputs:
+ * output[s] = fold of input over segment s with `op`; empty segments get
+ * *init (host pointer to one value of `dtype`), which is never folded into
+ * non-empty segments.  Integer sums wrap. */
+MGPU_HIP_API int mgpu_hip_segreduce(const void* input, int count,
+  const int* segments, int num_segments, void* output, int dtype, int op,
+  const void* init, void* workspace, size_t workspace_bytes,
+  mgpu_stream_t stream);
+
+/* Same, running only the selected phases (MGPU_PHASE_*).  A later phase uses
+ * what an earlier complete call left in the same workspace.  For timing the
+ * partition, tile and spine kernels separately. */
+MGPU_HIP_API int mgpu_hip_segreduce_phases(const void* input, int count,
+  const int* segments, int num_segments, void* output, int dtype, int op,
+  const void* init, void* workspace, size_t workspace_bytes,
+  mgpu_stream_t stream, int phases);
+
+/* mgpu::transform_segreduce (kernel_segreduce.hxx:272-280) with the functor
+ * of the reference's own test, f(index) = index % 13, int32 plus
+ * (tests/test_segreduce.cu:31-35).  Shows the generated-input path through
+ * the C ABI; arbitrary functors need the C++ templates. */
+MGPU_HIP_API int mgpu_hip_transform_segreduce_mod13(int count,
+  const int* segments, int num_segments, int* output, int init,
+  void* workspace, size_t workspace_bytes, mgpu_stream_t stream);
+
+/* mgpu::spmv (kernel_segreduce.hxx:285-298): CSR y = A * x.
+ * output[r] = sum over the row's nonzeros k of matrix[k] * vector[columns[k]];
+ * segments = row starts (num_segments rows, no trailing nnz entry);
+ * count = number of nonzeros; dtype MGPU_F32 or MGPU_F64; empty row => 0.
+ * Workspace: mgpu_hip_segreduce_workspace_bytes(count, num_segments, dtype). */
+MGPU_HIP_API int mgpu_hip_spmv(const void* matrix, const int* columns,
+  const void* vector, int count, const int* segments, int num_segments,
+  void* output, int dtype, void* workspace, size_t workspace_bytes,
+  mgpu_stream_t stream);
+MGPU_HIP_API int mgpu_hip_spmv_phases(const void* matrix, const int* columns,
+  const void* vector, int count, const int* segments, int num_segments,
+  void* output, int dtype, void* workspace, size_t workspace_bytes,
+  mgpu_stream_t stream, int phases);
+
+/* ---- load-balancing search --------------------------------------------- */
+
+/* Bytes of workspace the functions below need (the partition array). */
+MGPU_HIP_API size_t mgpu_hip_lbs_workspace_bytes(int count, int num_segments);
+
+/* mgpu::load_balance_search (kernel_load_balance.hxx:78-86):
+ * output[i] = index of the last segment whose start is <= i, i in [0,count). */
+MGPU_HIP_API int mgpu_hip_load_balance_search(int count, const int* segments,
+  int num_segments, int* output, void* workspace, size_t workspace_bytes,
+  mgpu_stream_t stream);
+MGPU_HIP_API int mgpu_hip_load_balance_search_phases(int count,
+  const int* segments, int num_segments, int* output, void* workspace,
+  size_t workspace_bytes, mgpu_stream_t stream, int phases);
+
+/* mgpu::transform_lbs (kernel_load_balance.hxx:8-76) with a functor that
+ * stores its arguments: seg_out[i] = segment of item i and
+ * rank_out[i] = i - segments[seg_out[i]].  Either output may be NULL. */
+MGPU_HIP_API int mgpu_hip_transform_lbs(int count, const int* segments,
+  int num_segments, int* seg_out, int* rank_out, void* workspace,
+  size_t workspace_bytes, mgpu_stream_t stream);
+
+/* mgpu::interval_expand (kernel_intervalmove.hxx:7-20):
+ * output[i] = input[segment of i] for elements of elem_bytes in
+ * {1, 2, 4, 8, 16} bytes (copied bit-for-bit). */
+MGPU_HIP_API int mgpu_hip_interval_expand(const void* input, int elem_bytes,
+  int count, const int* segments, int num_segments, void* output,
+  void* workspace, size_t workspace_bytes, mgpu_stream_t stream);
+MGPU_HIP_API int mgpu_hip_interval_expand_phases(const void* input,
+  int elem_bytes, int count, const int* segments, int num_segments,
+  void* output, void* workspace, size_t workspace_bytes,
+  mgpu_stream_t stream, int phases);
+
+/* mgpu::interval_gather (kernel_intervalmove.hxx:22-35):
+ * output[i] = input[gather[seg] + rank]. */
+MGPU_HIP_API int mgpu_hip_interval_gather(const void* input, int elem_bytes,
+  int count, const int* segments, int num_segments, const int* gather,
+  void* output, void* workspace, size_t workspace_bytes,
+  mgpu_stream_t stream);
+/* mgpu::interval_scatter (kernel_intervalmove.hxx:37-50):
+ * output[scatter[seg] + rank] = input[i]. */
+MGPU_HIP_API int mgpu_hip_interval_scatter(const void* input, int elem_bytes,
+  int count, const int* segments, int num_segments, const int* scatter,
+  void* output, void* workspace, size_t workspace_bytes,
+  mgpu_stream_t stream);
+/* mgpu::interval_move (kernel_intervalmove.hxx:52-65):
+ * output[scatter[seg] + rank] = input[gather[seg] + rank]. */
+MGPU_HIP_API int mgpu_hip_interval_move(const void* input, int elem_bytes,
+  int count, const int* segments, int num_segments, const int* scatter,
+  const int* gather, void* output, void* workspace, size_t workspace_bytes,
+  mgpu_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* MGPU_HIP_H */

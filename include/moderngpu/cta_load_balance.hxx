@@ -1,0 +1,305 @@
+// mgpu for AMD CDNA4: the CTA-level load-balancing search.
+//
+// A tile is nv = nt * vt consecutive elements of the merge of work-item
+// indices (A) with segment starts (B); the partition kernel supplies the
+// split, so a tile holds a_count items and b_count segment starts with
+// a_count + b_count <= nv, whatever the skew of the segment lengths.
+//
+// How the tile is decoded here differs from the CUDA library this API
+// mirrors (src/moderngpu/cta_load_balance.hxx:16-184).  That code gives each
+// thread one cross-diagonal, finds it with a binary search in shared memory
+// and then walks vt + 1 dependent shared-memory compares.  On CDNA that chain
+// of dependent LDS reads is latency bound, so this implementation does:
+//   1. zero an int marker per item slot in LDS (16-byte stores);
+//   2. every segment that owns at least one item of the tile writes
+//      (its index in the tile + 1) at the slot of its first item -- one plain
+//      LDS store per segment, no atomics, because among equal starts only the
+//      last one owns items;
+//   3. each thread max-scans vt consecutive slots in registers (independent
+//      16-byte LDS reads), one cta_scan_t<max> over the thread totals carries
+//      the running segment across threads, and the result is written back;
+//   4. the slots are read back in strided order, which is the coalesced order
+//      for whatever the caller stores per item.
+// The LDS layout pads one 16-byte chunk after every eight so that both the
+// strided and the thread-order 16-byte accesses spread over all banks.
+#pragma once
+#include "cta_merge.hxx"
+#include "cta_scan.hxx"
+#include "operators.hxx"
+#include "cpp11.hxx"
+
+BEGIN_MGPU_NAMESPACE
+
+namespace detail {
+
+////////////////////////////////////////////////////////////////////////////////
+// 16-byte vectors of W elements; the _u form may sit at any element-aligned
+// address in global memory (global_load/store_dwordx4 only need dword
+// alignment).
+
+template<typename type_t, int W>
+struct vec_t {
+  typedef type_t type __attribute__((ext_vector_type(W)));
+  typedef type_t type_u __attribute__((ext_vector_type(W),
+    aligned(sizeof(type_t))));
+};
+
+// Tile element p lives at LDS element index(p).  W = elements per 16-byte
+// chunk (1 disables chunking and padding).
+template<int W>
+struct tile_layout_t {
+  MGPU_HOST_DEVICE static constexpr int index(int p) {
+    return W > 1 ? p + (p / (8 * W)) * W : p;
+  }
+  MGPU_HOST_DEVICE static constexpr int capacity(int n) {
+    return index(n) + 2 * W;
+  }
+};
+
+// Elements per 16-byte chunk when the tile of vt values per thread can be
+// moved in whole chunks, else 1.
+template<typename type_t, int vt>
+struct chunk_width_t {
+  enum {
+    can = std::is_arithmetic<type_t>::value &&
+      (sizeof(type_t) == 4 || sizeof(type_t) == 8) &&
+      0 == vt % (16 / sizeof(type_t)),
+    value = can ? 16 / sizeof(type_t) : 1
+  };
+};
+
+// Read W consecutive LDS elements starting at an index that is a multiple
+// of W.
+template<int W, typename type_t>
+MGPU_DEVICE inline void lds_load_chunk(const type_t* p, type_t (&x)[W]) {
+  if(W > 1) {
+    typedef typename vec_t<type_t, (W > 1 ? W : 2)>::type v_t;
+    v_t v = *(const v_t*)p;
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) x[e] = v[e];
+  } else
+    x[0] = p[0];
+}
+template<int W, typename type_t>
+MGPU_DEVICE inline void lds_store_chunk(type_t* p, const type_t (&x)[W]) {
+  if(W > 1) {
+    typedef typename vec_t<type_t, (W > 1 ? W : 2)>::type v_t;
+    v_t v;
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) v[e] = x[e];
+    *(v_t*)p = v;
+  } else
+    p[0] = x[0];
+}
+
+} // namespace detail
+
+////////////////////////////////////////////////////////////////////////////////
+
+// Kept for source compatibility: where a thread's slice of the merge starts.
+struct lbs_placement_t {
+  merge_range_t range;    // range of loaded values
+  int a_index;            // first item of the thread
+  int b_index;            // segment of that item
+};
+
+template<int nt, int vt>
+struct cta_load_balance_t {
+  enum {
+    nv = nt * vt,
+    W = detail::chunk_width_t<int, vt>::value,
+    chunks = vt / W
+  };
+  typedef detail::tile_layout_t<W> layout_t;
+  typedef cta_scan_t<nt, int> scan_t;
+
+  struct storage_t {
+    // Item slots (padded layout), then the tile's segment starts:
+    // starts[0] belongs to the segment that is open when the tile begins,
+    // starts[1 + j] to segment b_begin + j.
+    alignas(16) int indices[layout_t::capacity(nv) + 4];
+    typename scan_t::storage_t scan;
+  };
+
+  struct result_t {
+    lbs_placement_t placement;
+    merge_range_t merge_range;
+    int merge_flags;                // not produced by this implementation
+
+    // Strided order: element i is tile item nt * i + tid.
+    array_t<int, vt> indices;       // global item index
+    array_t<int, vt> segments;      // segment of the item
+    array_t<int, vt> ranks;         // item index - start of its segment
+  };
+
+  // Index of the first start slot for a tile with a_count items.
+  MGPU_DEVICE static int starts_offset(int a_count) {
+    return layout_t::index((a_count + W - 1) / W * W) + W;
+  }
+
+  // Decodes the tile and leaves, for every item slot p in [0, a_count),
+  // (segment of item - (b_begin - 1)) in storage.indices[index(p)], and the
+  // segment starts behind them.  Ends with a barrier.
+  template<typename segments_it, typename partition_it>
+  MGPU_DEVICE merge_range_t fill(int count, segments_it segments,
+    int num_segments, int tid, int cta, partition_it partitions,
+    storage_t& storage) const {
+
+    merge_range_t range = compute_merge_range(count, num_segments, cta, nv,
+      partitions[cta], partitions[cta + 1]);
+    int a_count = range.a_count();
+    int b_count = range.b_count();
+    int* slots = storage.indices;
+    int* starts = storage.indices + starts_offset(a_count);
+
+    // 1. clear the item slots.
+    int zero[W];
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) zero[e] = 0;
+    PRAGMA_UNROLL
+    for(int i = 0; i < chunks; ++i) {
+      int p = W * (nt * i + tid);
+      if(p < a_count)
+        detail::lds_store_chunk<W>(slots + layout_t::index(p), zero);
+    }
+
+    // 2. stage the segment starts of the tile.
+    for(int j = tid; j < b_count; j += nt)
+      starts[1 + j] = segments[range.b_begin + j];
+    if(!tid) starts[0] = range.b_begin ? segments[range.b_begin - 1] : 0;
+    __syncthreads();
+
+    // 3. one marker per segment that owns items here.  Starts ascend, so
+    // among equal starts only the last segment is non-empty; a start at or
+    // past a_end owns nothing in this tile.
+    for(int j = tid; j < b_count; j += nt) {
+      int s0 = starts[1 + j];
+      int s1 = (j + 1 < b_count) ? starts[2 + j] : 0x7fffffff;
+      int p = s0 - range.a_begin;
+      if(s0 != s1 && p >= 0 && p < a_count)
+        slots[layout_t::index(p)] = j + 1;
+    }
+    __syncthreads();
+
+    // 4. running maximum along the items: vt slots per thread in registers,
+    // one exclusive max-scan over the thread totals.
+    int x[vt];
+    PRAGMA_UNROLL
+    for(int c = 0; c < chunks; ++c) {
+      int chunk[W];
+      detail::lds_load_chunk<W>(
+        slots + layout_t::index(vt * tid + W * c), chunk);
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) x[W * c + e] = chunk[e];
+    }
+    PRAGMA_UNROLL
+    for(int i = 1; i < vt; ++i) x[i] = max(x[i - 1], x[i]);
+
+    scan_result_t<int> carry = scan_t().scan(tid, x[vt - 1], storage.scan,
+      nt, maximum_t<int>(), 0, scan_type_exc);
+
+    PRAGMA_UNROLL
+    for(int c = 0; c < chunks; ++c) {
+      int chunk[W];
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) chunk[e] = max(carry.scan, x[W * c + e]);
+      // Slots at or past a_count belong to the segment starts: leave them.
+      if(vt * tid + W * c < a_count)
+        detail::lds_store_chunk<W>(
+          slots + layout_t::index(vt * tid + W * c), chunk);
+    }
+    __syncthreads();
+    return range;
+  }
+
+  // Full search: (index, segment, rank) per item in strided order.  Items
+  // past the end of the tile get segment b_begin and rank -1.
+  template<typename segments_it, typename partition_it>
+  MGPU_DEVICE result_t load_balance(int count, segments_it segments,
+    int num_segments, int tid, int cta, partition_it partitions,
+    storage_t& storage) const {
+
+    merge_range_t range = fill(count, segments, num_segments, tid, cta,
+      partitions, storage);
+    int a_count = range.a_count();
+    const int* slots = storage.indices;
+    const int* starts = storage.indices + starts_offset(a_count);
+
+    result_t result;
+    result.merge_range = range;
+    result.placement = lbs_placement_t { range, range.a_begin,
+      range.b_begin - 1 };
+    result.merge_flags = 0;
+    iterate<vt>([&](int i) {
+      int j = nt * i + tid;
+      result.indices[i] = range.a_begin + j;
+      if(j < a_count) {
+        int rel = slots[layout_t::index(j)];
+        result.segments[i] = range.b_begin - 1 + rel;
+        result.ranks[i] = result.indices[i] - starts[rel];
+      } else {
+        result.segments[i] = range.b_begin;
+        result.ranks[i] = -1;
+      }
+    });
+    __syncthreads();
+    return result;
+  }
+};
+
+namespace detail {
+
+////////////////////////////////////////////////////////////////////////////////
+// Per-segment values ("caching iterators") for the items of a tile.  When the
+// tile touches at most nt segments each value is read from global memory once
+// and fanned out through LDS; otherwise every item gathers its own
+// (interface after src/moderngpu/cta_load_balance.hxx:189-259).
+
+template<int nt, typename pointers_t>
+struct cached_segment_load_t {
+  enum { size = tuple_size<pointers_t>::value };
+  typedef tuple_iterator_value_t<pointers_t> value_t;
+
+  struct storage_t {
+    value_t data[nt];
+  };
+
+  // range = segments the tile's items can belong to.
+  template<int vt0, int vt>
+  MGPU_DEVICE static array_t<value_t, vt> load(int tid, int count,
+    range_t range, array_t<int, vt> segments, storage_t& storage,
+    pointers_t iterators) {
+
+    array_t<value_t, vt> loaded;
+    if(range.count() <= nt) {
+      if(tid < range.count() && range.begin + tid >= 0)
+        storage.data[tid] = mgpu::load(iterators, range.begin + tid);
+      __syncthreads();
+      strided_iterate<nt, vt, vt0>([&](int i, int) {
+        loaded[i] = storage.data[segments[i] - range.begin];
+      }, tid, count);
+      __syncthreads();
+    } else {
+      strided_iterate<nt, vt, vt0>([&](int i, int) {
+        loaded[i] = mgpu::load(iterators, segments[i]);
+      }, tid, count);
+    }
+    return loaded;
+  }
+};
+
+template<int nt>
+struct cached_segment_load_t<nt, tuple<> > {
+  typedef empty_t storage_t;
+  typedef tuple<> value_t;
+
+  template<int vt0, int vt>
+  MGPU_DEVICE static array_t<value_t, vt> load(int, int, range_t,
+    array_t<int, vt>, storage_t&, tuple<>) {
+    return array_t<value_t, vt>();
+  }
+};
+
+} // namespace detail
+
+END_MGPU_NAMESPACE

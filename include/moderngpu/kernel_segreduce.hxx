@@ -1,0 +1,512 @@
+// mgpu for AMD CDNA4: segmented reduction, transform_segreduce and CSR spmv.
+//
+//   output[s] = input[segments[s]] op ... op input[segments[s + 1] - 1]
+// (the last segment ends at count); an empty segment yields init and init is
+// not folded into non-empty ones.  segments[0] must be 0, starts ascend.
+// Public interface after src/moderngpu/kernel_segreduce.hxx:193-298.
+//
+// Structure (three kinds of kernel on the context's stream):
+//   K1  load_balance_partitions cuts the merge of items and segment starts
+//       into tiles of nv merged elements (search.hxx).
+//   K2  segreduce_tile_f: one CTA per tile.
+//         - the tile's items are fetched with 16-byte loads in strided order
+//           (unaligned starts are fine for global_load_dwordx4) and written
+//           to LDS in a padded thread-order layout;
+//         - meanwhile the tile's segment starts set one bit per start in an
+//           LDS bitmask (ds_or_b32);
+//         - each thread runs a flag-driven inclusive segmented scan over its
+//           vt consecutive items in registers and writes the scanned values
+//           back in place, so LDS slot e now holds the fold of its segment
+//           from max(segment start, thread start) to e;
+//         - one cta_segscan_t over the thread totals gives every thread the
+//           fold that flows into it;
+//         - one thread per segment start then picks the slot where its
+//           segment ends in the tile, adds the flow into that slot's thread if
+//           the segment began in an earlier thread, and stores output[s].
+//       The segment that was already open when the tile began is reported as
+//       a (segment, partial) carry for the spine.
+//   K3  segreduce_spine_f folds the per-tile carries of segments that span
+//       tiles into output[]; 1024 carries per CTA, repeated on the per-CTA
+//       carries until one CTA is left.
+// The CUDA reference instead walks vt + 1 merged elements per thread through
+// dependent shared-memory reads and keeps an "overwrite" bit per tile; here
+// the spine decides between combine and overwrite by comparing the segment's
+// start with the first item of the tile that carried it.
+#pragma once
+#include "search.hxx"
+#include "cta_load_balance.hxx"
+#include "cta_segscan.hxx"
+#include "transform.hxx"
+#include "memory.hxx"
+
+BEGIN_MGPU_NAMESPACE
+
+namespace detail {
+
+////////////////////////////////////////////////////////////////////////////////
+// Loading W consecutive tile items.  Raw pointers to 4/8-byte arithmetic
+// types use one (possibly unaligned) 16-byte global load; anything else is
+// element-wise through operator[].
+
+template<typename input_it, typename type_t, int W>
+struct tile_loader_t {
+  MGPU_DEVICE static void load(input_it input, int index, type_t (&x)[W]) {
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) x[e] = input[index + e];
+  }
+};
+
+template<typename type_t, int W>
+struct pointer_loader_t {
+  MGPU_DEVICE static void load(const type_t* input, int index,
+    type_t (&x)[W]) {
+    if(W > 1) {
+      typedef typename vec_t<type_t, (W > 1 ? W : 2)>::type_u v_t;
+      v_t v = *(const v_t*)(input + index);
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) x[e] = v[e];
+    } else
+      x[0] = input[index];
+  }
+};
+template<typename type_t, int W>
+struct tile_loader_t<const type_t*, type_t, W> : pointer_loader_t<type_t, W> { };
+template<typename type_t, int W>
+struct tile_loader_t<type_t*, type_t, W> : pointer_loader_t<type_t, W> { };
+
+// The fused spmv load: matrix[k] * vector[columns[k]], with the matrix values
+// and column indices of W consecutive nonzeros fetched as 16-byte loads.
+template<typename type_t>
+struct spmv_input_t {
+  typedef type_t value_type;
+  const type_t* matrix;
+  const int* columns;
+  const type_t* vector;
+  MGPU_DEVICE type_t operator[](int k) const {
+    return matrix[k] * vector[columns[k]];
+  }
+};
+template<typename type_t, int W>
+struct tile_loader_t<spmv_input_t<type_t>, type_t, W> {
+  MGPU_DEVICE static void load(spmv_input_t<type_t> in, int index,
+    type_t (&x)[W]) {
+    type_t a[W];
+    int c[W];
+    pointer_loader_t<type_t, W>::load(in.matrix, index, a);
+    // Columns are 4-byte: W of them are 16 bytes or less.
+    if(W > 1) {
+      typedef typename vec_t<int, (W > 1 ? W : 2)>::type_u v_t;
+      v_t v = *(const v_t*)(in.columns + index);
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) c[e] = v[e];
+    } else
+      c[0] = in.columns[index];
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) x[e] = a[e] * in.vector[c[e]];
+  }
+};
+
+////////////////////////////////////////////////////////////////////////////////
+// Default tiles on gfx950, by value size.
+
+template<typename type_t>
+struct segreduce_launch_default_t {
+  typedef launch_box_t<
+    arch_gfx950_cta<256, (sizeof(type_t) > 4 ? 8 : 16)>
+  > type_t_;
+};
+
+////////////////////////////////////////////////////////////////////////////////
+// K2
+
+template<typename launch_t, typename input_it, typename segments_it,
+  typename output_it, typename op_t, typename type_t>
+struct segreduce_tile_f {
+  input_it input;
+  int count;
+  segments_it segments;
+  int num_segments;
+  output_it output;
+  op_t op;
+  type_t init;
+  const int* mp_data;
+  type_t* carry_values;
+  int* carry_codes;
+
+  MGPU_DEVICE void operator()(int tid, int cta) const {
+    typedef typename launch_t::sm_ptx params_t;
+    enum {
+      nt = params_t::nt, vt = params_t::vt, nv = nt * vt,
+      W = chunk_width_t<type_t, vt>::value,
+      chunks = vt / W,
+      flag_words = nv / 32 + 2
+    };
+    static_assert(vt <= 32, "segreduce tiles hold at most 32 values/thread");
+    typedef tile_layout_t<W> layout_t;
+    typedef cta_segscan_t<nt, type_t> segscan_t;
+    typedef tile_loader_t<input_it, type_t, W> loader_t;
+
+    __shared__ struct {
+      alignas(16) type_t values[layout_t::capacity(nv)];
+      type_t flow[nt];              // fold flowing into each thread
+      unsigned flags[flag_words];   // bit p: a segment starts at tile item p
+      typename segscan_t::storage_t segscan;
+    } shared;
+
+    merge_range_t range = compute_merge_range(count, num_segments, cta, nv,
+      mp_data[cta], mp_data[cta + 1]);
+    int a_count = range.a_count();
+    int b_count = range.b_count();
+
+    // Issue the item loads first; they are consumed after the flag setup.
+    type_t r[chunks][W];
+    PRAGMA_UNROLL
+    for(int i = 0; i < chunks; ++i) {
+      int p = W * (nt * i + tid);
+      if(p + W <= a_count)
+        loader_t::load(input, range.a_begin + p, r[i]);
+      else {
+        PRAGMA_UNROLL
+        for(int e = 0; e < W; ++e)
+          if(p + e < a_count) r[i][e] = input[range.a_begin + p + e];
+      }
+    }
+
+    for(int w = tid; w < flag_words; w += nt) shared.flags[w] = 0;
+    __syncthreads();
+
+    // One bit per segment start.  Starts of this tile lie in
+    // [a_begin, a_end]; the clamp only guards against malformed input.
+    int first_start = 0;
+    for(int j = tid; j < b_count; j += nt) {
+      int s = segments[range.b_begin + j];
+      if(j == tid) first_start = s;
+      int p = min(max(s - range.a_begin, 0), a_count);
+      atomicOr(&shared.flags[p >> 5], 1u << (p & 31));
+    }
+
+    PRAGMA_UNROLL
+    for(int i = 0; i < chunks; ++i) {
+      int p = W * (nt * i + tid);
+      if(p < a_count)
+        lds_store_chunk<W>(shared.values + layout_t::index(p), r[i]);
+    }
+    __syncthreads();
+
+    // Thread order: items [vt * tid, vt * tid + vt) and their start bits.
+    type_t x[vt];
+    PRAGMA_UNROLL
+    for(int c = 0; c < chunks; ++c) {
+      type_t chunk[W];
+      lds_load_chunk<W>(shared.values + layout_t::index(vt * tid + W * c),
+        chunk);
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) x[W * c + e] = chunk[e];
+    }
+    unsigned bits;
+    {
+      int pos = vt * tid;
+      unsigned long long two = shared.flags[pos >> 5] |
+        ((unsigned long long)shared.flags[(pos >> 5) + 1] << 32);
+      bits = (unsigned)(two >> (pos & 31));
+      if(vt < 32) bits &= (1u << vt) - 1;
+    }
+
+    // Inclusive segmented scan of the thread's items, left to right.
+    PRAGMA_UNROLL
+    for(int i = 1; i < vt; ++i)
+      x[i] = ((bits >> i) & 1) ? x[i] : op(x[i - 1], x[i]);
+
+    PRAGMA_UNROLL
+    for(int c = 0; c < chunks; ++c) {
+      type_t chunk[W];
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) chunk[e] = x[W * c + e];
+      if(vt * tid + W * c < a_count)
+        lds_store_chunk<W>(shared.values + layout_t::index(vt * tid + W * c),
+          chunk);
+    }
+
+    segscan_result_t<type_t> flow = segscan_t().segscan(tid, 0 != bits, true,
+      x[vt - 1], shared.segscan, init, op);
+    shared.flow[tid] = flow.scan;
+    __syncthreads();
+
+    // Fold of tile items [p .. e], where no segment starts inside (p, e].
+    auto fold_to = [&](int p, int e) -> type_t {
+      int te = e / vt;
+      type_t v = shared.values[layout_t::index(e)];
+      if(p < te * vt) v = op(shared.flow[te], v);
+      return v;
+    };
+
+    // One thread per segment start of the tile.
+    for(int j = tid; j < b_count; j += nt) {
+      int seg = range.b_begin + j;
+      int s = (j == tid) ? first_start : segments[seg];
+      int next = (seg + 1 < num_segments) ? segments[seg + 1] : count;
+      int p = s - range.a_begin;
+      if(next <= s) output[seg] = init;                  // empty segment
+      else if(p >= 0 && p < a_count) {
+        int e = min(next, range.a_end) - range.a_begin - 1;
+        output[seg] = fold_to(p, e);
+      }
+      // else: the segment's first item is in the next tile; the spine
+      // writes it.
+    }
+
+    // The segment that was open when the tile began owns items [0, f).
+    if(!tid) {
+      int f = a_count;
+      if(b_count) f = min(max(first_start - range.a_begin, 0), a_count);
+      if(f > 0 && range.b_begin > 0) {
+        carry_values[cta] = fold_to(-1, f - 1);
+        carry_codes[cta] = range.b_begin - 1;
+      } else {
+        carry_values[cta] = init;
+        carry_codes[cta] = -1;
+      }
+    }
+  }
+};
+
+////////////////////////////////////////////////////////////////////////////////
+// K3: fold carries into the output.  codes[i] = segment that tile i carried
+// into (-1: none); equal codes are consecutive.  A CTA handles nt carries;
+// the run that is already open at its first carry is passed on to the next
+// level as one carry per CTA.  At the first level tile_begin = the partition
+// array (first item of every tile) decides whether the segment already has a
+// value in output[] (its start tile held some of its items) or not.
+
+template<int nt, typename output_it, typename segments_it, typename op_t,
+  typename type_t>
+struct segreduce_spine_f {
+  output_it output;
+  const type_t* values;
+  const int* codes;
+  int n;
+  segments_it segments;
+  const int* tile_begin;       // null above the first level
+  op_t op;
+  type_t init;
+  type_t* values_out;
+  int* codes_out;
+
+  MGPU_DEVICE void operator()(int tid, int cta) const {
+    typedef cta_segscan_t<nt, type_t> segscan_t;
+    __shared__ typename segscan_t::storage_t shared;
+
+    int gid = nt * cta + tid;
+    int code = (gid < n) ? codes[gid] : -1;
+    int prev = (gid > 0 && gid - 1 < n) ? codes[gid - 1] : -1;
+    int next = (gid + 1 < n) ? codes[gid + 1] : -1;
+    type_t value = (gid < n) ? values[gid] : init;
+
+    bool head = code != prev || -1 == code;
+    bool carry_out = -1 != code && code == next;
+
+    segscan_result_t<type_t> result = segscan_t().segscan(tid, head,
+      carry_out, value, shared, init, op);
+
+    bool run_end = -1 != code && (!carry_out || nt - 1 == tid);
+    if(run_end) {
+      if(result.has_carry_in) value = op(result.scan, value);
+      if(result.has_left_head) {
+        // The run started inside this CTA at carry index first.
+        int first = nt * cta + result.left_lane;
+        bool fresh = tile_begin && segments[code] >= tile_begin[first];
+        output[code] = fresh ? value : op(output[code], value);
+      } else {
+        values_out[cta] = value;
+        codes_out[cta] = code;
+      }
+    }
+    // No open run at the CTA's first carry: nothing to pass on.
+    if(!tid && (head || -1 == code)) {
+      values_out[cta] = init;
+      codes_out[cta] = -1;
+    }
+  }
+};
+
+////////////////////////////////////////////////////////////////////////////////
+// Workspace layout for one segreduce call (device memory, 256-byte aligned
+// pieces): partitions, tile carries, then the carries of each spine level.
+
+struct segreduce_workspace_t {
+  enum { spine_nt = 1024, max_levels = 4 };
+  int num_ctas, num_partitions, levels;
+  int level_count[max_levels + 1];      // carries entering each level
+  size_t mp_offset, codes_offset[max_levels + 1],
+    values_offset[max_levels + 1], bytes;
+
+  static size_t align(size_t x) { return (x + 255) & ~(size_t)255; }
+
+  segreduce_workspace_t(int count, int num_segments, int nv,
+    size_t value_size) {
+    int64_t total = (int64_t)count + num_segments;
+    num_ctas = (int)((total + nv - 1) / nv);
+    num_partitions = num_ctas + 1;
+    size_t at = 0;
+    mp_offset = at; at = align(at + sizeof(int) * num_partitions);
+    levels = 0;
+    int n = num_ctas;
+    for(;;) {
+      level_count[levels] = n;
+      codes_offset[levels] = at; at = align(at + sizeof(int) * n);
+      values_offset[levels] = at; at = align(at + value_size * n);
+      if(n <= 1 || levels == max_levels) break;
+      n = (n + spine_nt - 1) / spine_nt;
+      ++levels;
+    }
+    bytes = at;
+  }
+};
+
+enum {
+  phase_partition = 1,    // K1
+  phase_tiles = 2,        // K2
+  phase_spine = 4,        // K3, all levels
+  phase_all = 7
+};
+
+// Launches K1, K2 and the spine into caller-provided workspace.  `phases`
+// selects a subset for measurement; a later phase then relies on what an
+// earlier full call left in the workspace.
+template<typename launch_t, typename input_it, typename segments_it,
+  typename output_it, typename op_t, typename type_t>
+void segreduce_launch(input_it input, int count, segments_it segments,
+  int num_segments, output_it output, op_t op, type_t init, void* workspace,
+  const segreduce_workspace_t& ws, context_t& context,
+  int phases = phase_all) {
+
+  if(!ws.num_ctas) return;
+  cta_dim_t cta_dim = launch_t::cta_dim(context);
+  char* base = (char*)workspace;
+  int* mp_data = (int*)(base + ws.mp_offset);
+
+  if(phases & phase_partition)
+    merge_path_partitions_into<bounds_upper>(counting_iterator_t<int>(0),
+      (int64_t)count, segments, (int64_t)num_segments, (int64_t)cta_dim.nv(),
+      less_t<int>(), mp_data, context);
+
+  if(phases & phase_tiles) {
+    segreduce_tile_f<launch_t, input_it, segments_it, output_it, op_t, type_t>
+      k_reduce { input, count, segments, num_segments, output, op, init,
+        mp_data, (type_t*)(base + ws.values_offset[0]),
+        (int*)(base + ws.codes_offset[0]) };
+    cta_launch<launch_t>(k_reduce, ws.num_ctas, context);
+  }
+
+  enum { spine_nt = segreduce_workspace_t::spine_nt };
+  for(int level = 0; (phases & phase_spine) && level < ws.levels; ++level) {
+    int n = ws.level_count[level];
+    segreduce_spine_f<spine_nt, output_it, segments_it, op_t, type_t>
+      k_spine { output, (const type_t*)(base + ws.values_offset[level]),
+        (const int*)(base + ws.codes_offset[level]), n, segments,
+        level ? (const int*)nullptr : mp_data, op, init,
+        (type_t*)(base + ws.values_offset[level + 1]),
+        (int*)(base + ws.codes_offset[level + 1]) };
+    cta_launch<spine_nt>(k_spine, div_up(n, (int)spine_nt), context);
+  }
+}
+
+} // namespace detail
+
+////////////////////////////////////////////////////////////////////////////////
+
+template<typename launch_arg_t = empty_t, typename input_it,
+  typename segments_it, typename output_it, typename op_t, typename type_t>
+void segreduce(input_it input, int count, segments_it segments,
+  int num_segments, output_it output, op_t op, type_t init,
+  context_t& context);
+
+template<typename launch_arg_t = empty_t, typename func_t,
+  typename segments_it, typename output_it, typename op_t, typename type_t>
+void transform_segreduce(func_t f, int count, segments_it segments,
+  int num_segments, output_it output, op_t op, type_t init,
+  context_t& context);
+
+namespace detail {
+
+// Generic iterators: the product is formed element by element.
+template<typename matrix_it, typename columns_it, typename vector_it,
+  typename segments_it, typename output_it, typename launch_arg_t>
+void spmv_dispatch(matrix_it matrix, columns_it columns, vector_it vector,
+  int count, segments_it segments, int num_segments, output_it output,
+  context_t& context, launch_arg_t) {
+  typedef typename std::iterator_traits<matrix_it>::value_type type_t;
+  transform_segreduce<launch_arg_t>([=]MGPU_DEVICE(int index) {
+    return matrix[index] * ldg(vector + columns[index]);
+  }, count, segments, num_segments, output, plus_t<type_t>(),
+    (type_t)0, context);
+}
+
+// Raw pointers: matrix values and column indices come in as 16-byte loads.
+template<typename type_t, typename segments_it, typename output_it,
+  typename launch_arg_t>
+void spmv_dispatch(const type_t* matrix, const int* columns,
+  const type_t* vector, int count, segments_it segments, int num_segments,
+  output_it output, context_t& context, launch_arg_t) {
+  segreduce<launch_arg_t>(spmv_input_t<type_t> { matrix, columns, vector },
+    count, segments, num_segments, output, plus_t<type_t>(), (type_t)0,
+    context);
+}
+template<typename type_t, typename segments_it, typename output_it,
+  typename launch_arg_t>
+void spmv_dispatch(type_t* matrix, int* columns, type_t* vector, int count,
+  segments_it segments, int num_segments, output_it output,
+  context_t& context, launch_arg_t) {
+  spmv_dispatch((const type_t*)matrix, (const int*)columns,
+    (const type_t*)vector, count, segments, num_segments, output, context,
+    launch_arg_t());
+}
+
+} // namespace detail
+
+template<typename launch_arg_t, typename input_it,
+  typename segments_it, typename output_it, typename op_t, typename type_t>
+void segreduce(input_it input, int count, segments_it segments,
+  int num_segments, output_it output, op_t op, type_t init,
+  context_t& context) {
+
+  typedef typename conditional_typedef_t<launch_arg_t,
+    typename detail::segreduce_launch_default_t<type_t>::type_t_
+  >::type_t launch_t;
+
+  cta_dim_t cta_dim = launch_t::cta_dim(context);
+  detail::segreduce_workspace_t ws(count, num_segments, cta_dim.nv(),
+    sizeof(type_t));
+  if(!ws.num_ctas) return;
+
+  mem_t<char> workspace(ws.bytes, context);
+  detail::segreduce_launch<launch_t>(input, count, segments, num_segments,
+    output, op, init, workspace.data(), ws, context);
+}
+
+// segreduce over values generated on the fly: input[i] = f(i).
+template<typename launch_arg_t, typename func_t,
+  typename segments_it, typename output_it, typename op_t, typename type_t>
+void transform_segreduce(func_t f, int count, segments_it segments,
+  int num_segments, output_it output, op_t op, type_t init,
+  context_t& context) {
+
+  segreduce<launch_arg_t>(make_load_iterator<type_t>(f), count, segments,
+    num_segments, output, op, init, context);
+}
+
+// CSR sparse matrix * dense vector.  segments = row starts (num_segments
+// entries, no trailing nnz), count = number of nonzeros.
+template<typename launch_arg_t = empty_t, typename matrix_it,
+  typename columns_it, typename vector_it, typename segments_it,
+  typename output_it>
+void spmv(matrix_it matrix, columns_it columns, vector_it vector,
+  int count, segments_it segments, int num_segments, output_it output,
+  context_t& context) {
+
+  typedef typename std::iterator_traits<matrix_it>::value_type type_t;
+  detail::spmv_dispatch(matrix, columns, vector, count, segments,
+    num_segments, output, context, launch_arg_t());
+}
+
+END_MGPU_NAMESPACE

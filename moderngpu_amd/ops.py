@@ -1,0 +1,252 @@
+"""Host-side mirror of the mgpu:: entry points on torch device tensors.
+
+Function names, argument meaning and error behaviour follow the reference
+templates (``segreduce``, ``spmv``, ``load_balance_search``, ``transform_lbs``,
+``interval_expand`` ..., see include/mgpu_hip.h for the file:line of each).
+Every call goes through the C ABI of libmgpu_hip.so and is enqueued on torch's
+current stream; nothing here computes on the CPU.
+"""
+import ctypes
+
+import torch
+
+from ._native import lib
+
+OPS = {"plus": 0, "maximum": 1, "minimum": 2}
+_DTYPES = {torch.int32: 0, torch.int64: 2, torch.float32: 4, torch.float64: 5}
+# torch has no uint32/uint64 arithmetic tensors worth using: unsigned values
+# travel as the same-width signed tensors with dtype_code overridden.
+_UNSIGNED = {"u32": (torch.int32, 1), "u64": (torch.int64, 3)}
+_CTYPE = {0: ctypes.c_int32, 1: ctypes.c_uint32, 2: ctypes.c_int64,
+          3: ctypes.c_uint64, 4: ctypes.c_float, 5: ctypes.c_double}
+
+
+class MgpuError(RuntimeError):
+    """A non-zero return code from libmgpu_hip (the C++ layer throws
+    cuda_exception_t in the same situations)."""
+
+    def __init__(self, code):
+        self.code = code
+        msg = lib().mgpu_hip_error_string(code)
+        super().__init__("libmgpu_hip error %d: %s" % (
+            code, msg.decode() if msg else "?"))
+
+
+def _check(code):
+    if code != 0:
+        raise MgpuError(code)
+
+
+def _ptr(t):
+    return ctypes.c_void_p(t.data_ptr()) if t is not None and t.numel() else None
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _dev_i32(t, name):
+    if t.dtype != torch.int32 or not t.is_cuda or not t.is_contiguous():
+        raise TypeError("%s must be a contiguous int32 CUDA tensor" % name)
+    return t
+
+
+_workspaces = {}
+
+
+def _workspace(nbytes, device):
+    """A per-device scratch tensor that only grows.  All calls run on the
+    current stream, so reuse between consecutive calls is ordered."""
+    key = (device.index, torch.cuda.current_stream().cuda_stream)
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < nbytes:
+        ws = torch.empty(max(int(nbytes), 1 << 16), dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def segreduce_tile_size(dtype_code):
+    return lib().mgpu_hip_segreduce_tile_size(dtype_code)
+
+
+def lbs_tile_size():
+    return lib().mgpu_hip_lbs_tile_size()
+
+
+def _dtype_code(t, unsigned):
+    if unsigned:
+        want, code = _UNSIGNED["u32" if t.dtype == torch.int32 else "u64"]
+        if t.dtype != want:
+            raise TypeError("unsigned values travel as int32/int64 tensors")
+        return code
+    if t.dtype not in _DTYPES:
+        raise TypeError("unsupported value type %s" % t.dtype)
+    return _DTYPES[t.dtype]
+
+
+def segreduce(values, segments, op="plus", init=0, out=None, unsigned=False,
+              phases=7, workspace=None):
+    """output[s] = fold of values over segment s; empty segments give init."""
+    _dev_i32(segments, "segments")
+    if not values.is_cuda or not values.is_contiguous():
+        raise TypeError("values must be a contiguous CUDA tensor")
+    code = _dtype_code(values, unsigned)
+    count, nseg = values.numel(), segments.numel()
+    if out is None:
+        out = torch.empty(nseg, dtype=values.dtype, device=values.device)
+    need = lib().mgpu_hip_segreduce_workspace_bytes(count, nseg, code)
+    ws = workspace if workspace is not None else _workspace(need, values.device)
+    init_c = _CTYPE[code](init)
+    _check(lib().mgpu_hip_segreduce_phases(
+        _ptr(values), count, _ptr(segments), nseg, _ptr(out), code, OPS[op],
+        ctypes.byref(init_c), _ptr(ws), ws.numel(), _stream(), phases))
+    return out
+
+
+def transform_segreduce_mod13(count, segments, init=-1, out=None):
+    """transform_segreduce with f(index) = index % 13, int32 plus."""
+    _dev_i32(segments, "segments")
+    nseg = segments.numel()
+    if out is None:
+        out = torch.empty(nseg, dtype=torch.int32, device=segments.device)
+    need = lib().mgpu_hip_segreduce_workspace_bytes(count, nseg, 0)
+    ws = _workspace(need, segments.device)
+    _check(lib().mgpu_hip_transform_segreduce_mod13(
+        count, _ptr(segments), nseg, _ptr(out), init, _ptr(ws), ws.numel(),
+        _stream()))
+    return out
+
+
+def spmv(matrix, columns, vector, segments, out=None, phases=7, workspace=None):
+    """CSR y = A x; segments are the row starts (no trailing nnz entry)."""
+    _dev_i32(segments, "segments")
+    _dev_i32(columns, "columns")
+    if matrix.dtype not in (torch.float32, torch.float64) or vector.dtype != matrix.dtype:
+        raise TypeError("matrix and vector must both be float32 or float64")
+    code = _DTYPES[matrix.dtype]
+    count, nseg = matrix.numel(), segments.numel()
+    if columns.numel() != count:
+        raise ValueError("columns and matrix differ in length")
+    if out is None:
+        out = torch.empty(nseg, dtype=matrix.dtype, device=matrix.device)
+    need = lib().mgpu_hip_segreduce_workspace_bytes(count, nseg, code)
+    ws = workspace if workspace is not None else _workspace(need, matrix.device)
+    _check(lib().mgpu_hip_spmv_phases(
+        _ptr(matrix), _ptr(columns), _ptr(vector), count, _ptr(segments), nseg,
+        _ptr(out), code, _ptr(ws), ws.numel(), _stream(), phases))
+    return out
+
+
+def load_balance_search(count, segments, out=None, phases=3, workspace=None):
+    """out[i] = last segment whose start is <= i."""
+    _dev_i32(segments, "segments")
+    nseg = segments.numel()
+    if out is None:
+        out = torch.empty(count, dtype=torch.int32, device=segments.device)
+    need = lib().mgpu_hip_lbs_workspace_bytes(count, nseg)
+    ws = workspace if workspace is not None else _workspace(need, segments.device)
+    _check(lib().mgpu_hip_load_balance_search_phases(
+        count, _ptr(segments), nseg, _ptr(out), _ptr(ws), ws.numel(),
+        _stream(), phases))
+    return out
+
+
+def transform_lbs(count, segments):
+    """(seg, rank) per work item, the arguments transform_lbs hands its functor."""
+    _dev_i32(segments, "segments")
+    nseg = segments.numel()
+    seg = torch.empty(count, dtype=torch.int32, device=segments.device)
+    rank = torch.empty(count, dtype=torch.int32, device=segments.device)
+    ws = _workspace(lib().mgpu_hip_lbs_workspace_bytes(count, nseg), segments.device)
+    _check(lib().mgpu_hip_transform_lbs(
+        count, _ptr(segments), nseg, _ptr(seg), _ptr(rank), _ptr(ws),
+        ws.numel(), _stream()))
+    return seg, rank
+
+
+def _lbs_ws(count, segments):
+    return _workspace(lib().mgpu_hip_lbs_workspace_bytes(count, segments.numel()),
+                      segments.device)
+
+
+def interval_expand(values, count, segments, out=None, phases=3, workspace=None):
+    """out[i] = values[segment of i]."""
+    _dev_i32(segments, "segments")
+    if values.numel() != segments.numel():
+        raise ValueError("one value per segment expected")
+    if out is None:
+        out = torch.empty(count, dtype=values.dtype, device=values.device)
+    ws = workspace if workspace is not None else _lbs_ws(count, segments)
+    _check(lib().mgpu_hip_interval_expand_phases(
+        _ptr(values), values.element_size(), count, _ptr(segments),
+        segments.numel(), _ptr(out), _ptr(ws), ws.numel(), _stream(), phases))
+    return out
+
+
+def interval_gather(inp, count, segments, gather, out=None):
+    """out[i] = inp[gather[seg] + rank]."""
+    _dev_i32(segments, "segments")
+    _dev_i32(gather, "gather")
+    if out is None:
+        out = torch.empty(count, dtype=inp.dtype, device=inp.device)
+    ws = _lbs_ws(count, segments)
+    _check(lib().mgpu_hip_interval_gather(
+        _ptr(inp), inp.element_size(), count, _ptr(segments), segments.numel(),
+        _ptr(gather), _ptr(out), _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
+def interval_scatter(inp, count, segments, scatter, out):
+    """out[scatter[seg] + rank] = inp[i]."""
+    _dev_i32(segments, "segments")
+    _dev_i32(scatter, "scatter")
+    ws = _lbs_ws(count, segments)
+    _check(lib().mgpu_hip_interval_scatter(
+        _ptr(inp), inp.element_size(), count, _ptr(segments), segments.numel(),
+        _ptr(scatter), _ptr(out), _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
+def interval_move(inp, count, segments, scatter, gather, out):
+    """out[scatter[seg] + rank] = inp[gather[seg] + rank]."""
+    _dev_i32(segments, "segments")
+    _dev_i32(scatter, "scatter")
+    _dev_i32(gather, "gather")
+    ws = _lbs_ws(count, segments)
+    _check(lib().mgpu_hip_interval_move(
+        _ptr(inp), inp.element_size(), count, _ptr(segments), segments.numel(),
+        _ptr(scatter), _ptr(gather), _ptr(out), _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
+def load_balance_partitions(count, segments, spacing):
+    """Merge-path splits every `spacing` merged elements (items + starts)."""
+    _dev_i32(segments, "segments")
+    n = lib().mgpu_hip_partition_count(count, segments.numel(), spacing)
+    out = torch.empty(n, dtype=torch.int32, device=segments.device)
+    _check(lib().mgpu_hip_load_balance_partitions(
+        count, _ptr(segments), segments.numel(), spacing, _ptr(out), _stream()))
+    return out
+
+
+def merge_path_partitions(a_keys, a_count, b_keys, spacing, bounds="lower"):
+    """Splits of the merge of two sorted int32 arrays (a_keys None = 0,1,2...)."""
+    _dev_i32(b_keys, "b_keys")
+    if a_keys is not None:
+        _dev_i32(a_keys, "a_keys")
+    n = lib().mgpu_hip_partition_count(a_count, b_keys.numel(), spacing)
+    out = torch.empty(n, dtype=torch.int32, device=b_keys.device)
+    _check(lib().mgpu_hip_merge_path_partitions(
+        _ptr(a_keys), a_count, _ptr(b_keys), b_keys.numel(), spacing,
+        1 if bounds == "upper" else 0, _ptr(out), _stream()))
+    return out
+
+
+def binary_search_partitions(keys, count, spacing, bounds="lower"):
+    _dev_i32(keys, "keys")
+    n = (count + spacing - 1) // spacing + 1
+    out = torch.empty(n, dtype=torch.int32, device=keys.device)
+    _check(lib().mgpu_hip_binary_search_partitions(
+        _ptr(keys), count, keys.numel(), spacing,
+        1 if bounds == "upper" else 0, _ptr(out), _stream()))
+    return out

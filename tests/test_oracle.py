@@ -1,0 +1,299 @@
+"""Pins the CPU oracle.  Every oracle function is checked against something
+that does not share its formula: vectors recorded from the reference's own
+host functions, the reference tests' expectations, closed forms, numpy/scipy
+library routines and brute force on small inputs."""
+import json
+import math
+import os
+
+import numpy as np
+import pytest
+
+from moderngpu_amd import workloads
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def _lengths(segments, count):
+    return np.diff(np.append(np.asarray(segments, dtype=np.int64), count))
+
+
+def _random_segments(rng, count, nseg, dup=0.3):
+    s = np.zeros(nseg, dtype=np.int32)
+    if nseg > 1:
+        draws = rng.integers(0, count + 1, size=nseg - 1)
+        if dup > 0 and nseg > 4:      # force runs of equal starts
+            k = max(1, int(dup * (nseg - 1)))
+            draws[rng.integers(0, nseg - 1, size=k)] = draws[rng.integers(0, nseg - 1, size=k)]
+        s[1:] = np.sort(draws)
+    return s
+
+
+# --- merge path / partitions -------------------------------------------------
+
+def test_merge_path_matches_reference_host_functions(oracle):
+    g = json.load(open(os.path.join(GOLDEN, "reference_host_functions.json")))
+    segs, count = g["segments"], g["count"]
+    got = [oracle.merge_path(None, count, segs, d) for d in range(count + len(segs) + 1)]
+    assert got == g["merge_path_upper_by_diag"]
+    assert list(oracle.compute_merge_range(*g["compute_merge_range"]["args"])) == \
+        g["compute_merge_range"]["result"]
+    b = g["binary_search"]
+    assert oracle.binary_search(b["keys"], b["key"], upper=False) == b["lower"]
+    assert oracle.binary_search(b["keys"], b["key"], upper=True) == b["upper"]
+
+
+def _explicit_merge_split(a, b, diag, upper):
+    """Brute force: really merge, count how many of the first diag came from A."""
+    i = j = 0
+    for _ in range(diag):
+        if j >= len(b):
+            take_a = True
+        elif i >= len(a):
+            take_a = False
+        else:
+            take_a = (a[i] < b[j]) if upper else (a[i] <= b[j])
+        if take_a:
+            i += 1
+        else:
+            j += 1
+    return i
+
+
+@pytest.mark.parametrize("upper", [True, False])
+def test_merge_path_brute_force(oracle, upper):
+    rng = np.random.default_rng(1)
+    for _ in range(60):
+        na, nb = int(rng.integers(0, 40)), int(rng.integers(0, 40))
+        a = np.sort(rng.integers(0, 25, size=na)).astype(np.int32)
+        b = np.sort(rng.integers(0, 25, size=nb)).astype(np.int32)
+        for diag in range(na + nb + 1):
+            want = _explicit_merge_split(a, b, diag, upper)
+            assert oracle.merge_path(a, na, b, diag, upper) == want
+
+
+def test_lbs_partition_invariants(oracle):
+    rng = np.random.default_rng(2)
+    for _ in range(20):
+        count = int(rng.integers(0, 5000))
+        nseg = int(rng.integers(1, 600))
+        segs = _random_segments(rng, count, nseg)
+        spacing = int(rng.integers(1, 300))
+        mp = oracle.lbs_partitions(count, segs, spacing)
+        total = count + nseg
+        assert mp.size == (total + spacing - 1) // spacing + 1
+        assert mp[0] == 0 and mp[-1] == count
+        assert np.all(np.diff(mp) >= 0)
+        for i, a in enumerate(mp):
+            diag = min(spacing * i, total)
+            b = diag - a
+            assert 0 <= b <= nseg
+            if b > 0:
+                assert segs[b - 1] <= a          # consumed starts are <= item
+            if b < nseg and a > 0:
+                assert a - 1 < segs[b]           # next start is after item a-1
+
+
+def test_binary_search_matches_numpy(oracle):
+    rng = np.random.default_rng(3)
+    keys = np.sort(rng.integers(0, 100, size=500)).astype(np.int32)
+    for key in range(-2, 103):
+        assert oracle.binary_search(keys, key, upper=False) == np.searchsorted(keys, key, "left")
+        assert oracle.binary_search(keys, key, upper=True) == np.searchsorted(keys, key, "right")
+    got = oracle.binary_search_partitions(keys, 100, 7, upper=False)
+    want = np.searchsorted(keys, np.minimum(np.arange(got.size) * 7, 100), "left")
+    assert np.array_equal(got, want)
+
+
+# --- load-balancing search ---------------------------------------------------
+
+def test_lbs_reference_test_vector(oracle):
+    # moderngpu tests/test_load_balance.cu:9-28: starts every 100, N = 200030.
+    count, spacing = 200030, 100
+    segs = np.arange(0, count, spacing, dtype=np.int32)
+    assert segs.size == (count + spacing - 1) // spacing
+    got = oracle.load_balance_search(count, segs)
+    assert np.array_equal(got, np.arange(count) // spacing)
+
+
+def test_lbs_closed_form_and_ranks(oracle):
+    rng = np.random.default_rng(4)
+    for _ in range(30):
+        count = int(rng.integers(0, 3000))
+        segs = _random_segments(rng, count, int(rng.integers(1, 400)))
+        seg, rank = oracle.transform_lbs(count, segs)
+        want = np.searchsorted(segs, np.arange(count), side="right") - 1
+        assert np.array_equal(seg, want)
+        assert np.array_equal(rank, np.arange(count) - segs[want])
+
+
+def test_interval_expand_is_repeat(oracle):
+    rng = np.random.default_rng(5)
+    for dtype in (np.int32, np.int64, np.uint8, np.float64):
+        count = 2500
+        segs = _random_segments(rng, count, 300)
+        vals = rng.integers(0, 200, size=300).astype(dtype)
+        got = oracle.interval_expand(vals, count, segs)
+        assert np.array_equal(got, np.repeat(vals, _lengths(segs, count)))
+
+
+def test_interval_gather_scatter_move(oracle):
+    rng = np.random.default_rng(6)
+    count, nseg = 1200, 90
+    segs = _random_segments(rng, count, nseg, dup=0.0)
+    lens = _lengths(segs, count)
+    # disjoint destination intervals: a shuffled packing of the segments.
+    order = rng.permutation(nseg)
+    dest = np.zeros(nseg, dtype=np.int64)
+    dest[order] = np.concatenate([[0], np.cumsum(lens[order])[:-1]])
+    dest = dest.astype(np.int32)
+    src = rng.integers(0, 10 ** 6, size=count).astype(np.int32)
+    seg = np.repeat(np.arange(nseg), lens)
+    rank = np.arange(count) - segs[seg]
+    assert np.array_equal(oracle.interval_gather(src, count, segs, dest), src[dest[seg] + rank])
+    want = np.zeros(count, dtype=np.int32)
+    want[dest[seg] + rank] = src
+    assert np.array_equal(oracle.interval_scatter(src, count, segs, dest, count), want)
+    gather = dest[::-1].copy()       # any valid source offsets of equal lengths
+    lens_r = lens
+    ok = gather.astype(np.int64) + lens_r <= count
+    gather[~ok] = 0
+    want = np.zeros(count, dtype=np.int32)
+    want[dest[seg] + rank] = src[gather[seg] + rank]
+    assert np.array_equal(oracle.interval_move(src, count, segs, dest, gather, count), want)
+
+
+# --- segmented reduce --------------------------------------------------------
+
+def test_segreduce_mod13_golden(oracle):
+    g = json.load(open(os.path.join(GOLDEN, "segreduce_mod13.json")))
+    for c in g["cases"]:
+        segs = np.array(c["segments"], dtype=np.int32)
+        want = np.array(c["expected"], dtype=np.int64)
+        got = oracle.segreduce_mod13(c["count"], segs, init=g["init"])
+        assert np.array_equal(got, want), c["seed"]
+        vals = (np.arange(c["count"]) % 13).astype(np.int32)
+        got2 = oracle.segreduce(vals, segs, "plus", g["init"])
+        assert np.array_equal(got2, want), c["seed"]
+
+
+def _numpy_segreduce(vals, segs, ufunc, init):
+    count = vals.size
+    lens = _lengths(segs, count)
+    out = np.full(segs.size, init, dtype=vals.dtype)
+    nz = lens > 0
+    if nz.any():
+        red = ufunc.reduceat(vals, segs[nz].astype(np.int64))
+        out[nz] = red
+    return out
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.uint32, np.int64, np.uint64])
+def test_segreduce_integers_vs_numpy(oracle, dtype):
+    rng = np.random.default_rng(7)
+    info = np.iinfo(dtype)
+    for _ in range(10):
+        count = int(rng.integers(1, 4000))
+        segs = _random_segments(rng, count, int(rng.integers(1, 300)))
+        vals = rng.integers(info.min, info.max, size=count, dtype=dtype, endpoint=True)
+        with np.errstate(over="ignore"):
+            assert np.array_equal(oracle.segreduce(vals, segs, "plus", 17),
+                                  _numpy_segreduce(vals, segs, np.add, 17))
+        assert np.array_equal(oracle.segreduce(vals, segs, "maximum", 3),
+                              _numpy_segreduce(vals, segs, np.maximum, 3))
+        assert np.array_equal(oracle.segreduce(vals, segs, "minimum", 5),
+                              _numpy_segreduce(vals, segs, np.minimum, 5))
+
+
+@pytest.mark.parametrize("dtype,tol", [(np.float32, 1e-5), (np.float64, 1e-12)])
+def test_segreduce_float_vs_fsum(oracle, dtype, tol):
+    rng = np.random.default_rng(8)
+    count = 3000
+    segs = _random_segments(rng, count, 120)
+    vals = rng.random(count).astype(dtype)
+    got = oracle.segreduce(vals, segs, "plus", -2.0)
+    lens = _lengths(segs, count)
+    for s in range(segs.size):
+        if lens[s] == 0:
+            assert got[s] == dtype(-2.0)
+        else:
+            exact = math.fsum(float(v) for v in vals[segs[s]:segs[s] + lens[s]])
+            # serial summation bound: (terms) * eps * sum|x|, well inside tol
+            # for these lengths (values are non-negative so sum|x| = exact).
+            assert abs(got[s] - exact) <= lens[s] * np.finfo(dtype).eps * abs(exact)
+            assert abs(got[s] - exact) <= tol * abs(exact) * max(1, lens[s] // 64 + 1)
+    assert np.array_equal(oracle.segreduce(vals, segs, "maximum", -1.0),
+                          _numpy_segreduce(vals, segs, np.maximum, dtype(-1.0)))
+    assert np.array_equal(oracle.segreduce(vals, segs, "minimum", 9.0),
+                          _numpy_segreduce(vals, segs, np.minimum, dtype(9.0)))
+
+
+def test_segreduce_brute_force_and_init_rule(oracle):
+    vals = np.array([5, 1, 4, 2, 8, 7], dtype=np.int32)
+    segs = np.array([0, 0, 2, 2, 2, 5, 6, 6], dtype=np.int32)
+    # segments: [], [5,1], [], [], [4,2,8], [7], [], []  -- init only in empties
+    assert list(oracle.segreduce(vals, segs, "plus", -100)) == \
+        [-100, 6, -100, -100, 14, 7, -100, -100]
+    assert list(oracle.segreduce(vals, segs, "maximum", -100)) == \
+        [-100, 5, -100, -100, 8, 7, -100, -100]
+    assert list(oracle.segreduce(vals, segs, "minimum", 100)) == \
+        [100, 1, 100, 100, 2, 7, 100, 100]
+
+
+def test_max_min_tie_rule_signed_zero(oracle):
+    # mgpu::max(a,b) = (a<b)?b:a keeps the left operand on ties.
+    vals = np.array([0.0, -0.0, -0.0, 0.0], dtype=np.float32)
+    segs = np.array([0, 2], dtype=np.int32)
+    mx = oracle.segreduce(vals, segs, "maximum", 0.0)
+    mn = oracle.segreduce(vals, segs, "minimum", 0.0)
+    assert list(np.signbit(mx)) == [False, True]
+    assert list(np.signbit(mn)) == [False, True]
+
+
+# --- spmv ----------------------------------------------------------------------
+
+def test_spmv_vs_scipy(oracle):
+    import scipy.sparse as sp
+    w = workloads.config4(seed=3, scale=4096)
+    rows = w["segments"].size
+    indptr = np.append(w["segments"].astype(np.int64), w["nnz"])
+    lens = _lengths(w["segments"], w["nnz"])
+    for dtype in (np.float32, np.float64):
+        # The oracle adds serially in `dtype`: its distance from the exact
+        # product is bounded by (terms + 1) * eps * sum|a x| (standard forward
+        # bound for recursive summation, products rounded once).
+        tol = (lens + 2) * np.finfo(dtype).eps
+        m = w["matrix"].astype(dtype)
+        x = w["vector"].astype(dtype)
+        # scipy canonicalises index arrays in place: hand it copies.
+        a = sp.csr_matrix((m.astype(np.float64), w["columns"].copy(), indptr.copy()),
+                          shape=(rows, rows))
+        want = a @ x.astype(np.float64)
+        abs_a = sp.csr_matrix((np.abs(m.astype(np.float64)), w["columns"].copy(),
+                               indptr.copy()), shape=(rows, rows))
+        norm = abs_a @ np.abs(x.astype(np.float64))
+        got = oracle.spmv(m, w["columns"], x, w["segments"])
+        assert got.dtype == dtype
+        assert np.all(np.abs(got - want) <= tol * norm + 1e-300)
+        assert np.allclose(oracle.spmv_abs(m, w["columns"], x, w["segments"]), norm, rtol=1e-12)
+
+
+def test_spmv_empty_rows_are_zero(oracle):
+    m = np.array([2.0, 3.0], dtype=np.float32)
+    c = np.array([1, 0], dtype=np.int32)
+    x = np.array([10.0, 100.0], dtype=np.float32)
+    segs = np.array([0, 0, 1, 2, 2], dtype=np.int32)
+    assert list(oracle.spmv(m, c, x, segs)) == [0.0, 200.0, 30.0, 0.0, 0.0]
+
+
+# --- scans ---------------------------------------------------------------------
+
+def test_scan_vs_numpy(oracle):
+    rng = np.random.default_rng(9)
+    v = rng.integers(-50, 50, size=777).astype(np.int32)
+    out, red = oracle.scan(v, "plus", 0, inclusive=True)
+    assert np.array_equal(out, np.cumsum(v)) and red == v.sum()
+    out, red = oracle.scan(v, "plus", 9, inclusive=False)
+    assert out[0] == 9 and np.array_equal(out[1:], np.cumsum(v)[:-1])
+    out, red = oracle.scan(v, "maximum", 0, inclusive=True)
+    assert np.array_equal(out, np.maximum.accumulate(v))
