@@ -1,0 +1,373 @@
+#!/usr/bin/env python3
+"""Benchmark of the segmented-reduce / load-balancing-search path on one
+MI355X.
+
+One "step" is one complete call of the hot path (partition kernel, tile
+kernel, carry spine) on a batch that is already resident in HBM.  The default
+workload is BASELINE.json's configs[1]: segmented fp32 sum over 2^26 values in
+2^20 geometric-length segments.  Inputs rotate over several independent copies
+so that the 256 MB memory-side cache cannot serve a 256 MiB input.
+
+Prints ONE JSON line (see the keys at the bottom).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E, published
+
+
+def _dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+class Workload:
+    """name, algorithmic bytes/items per step, device copies, step(i),
+    tiles(i) (dominant kernel only), parity check and CPU baseline."""
+
+
+def make_c2(copies):
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    w = workloads.config2()
+    n, s = w["values"].size, w["segments"].size
+    segs = [_dev(w["segments"]) for _ in range(copies)]
+    vals = [_dev(w["values"])]
+    for c in range(1, copies):          # independent values per copy
+        vals.append(torch.rand(n, dtype=torch.float32, device="cuda"))
+    outs = [torch.empty(s, dtype=torch.float32, device="cuda") for _ in range(copies)]
+    wk = Workload()
+    wk.name = "segreduce fp32 plus, 2^26 values, 2^20 geometric segments (mean 64, ~5% empty)"
+    wk.key = "c2_segreduce_f32"
+    wk.dtype = "f32"
+    wk.items = n
+    wk.bytes = n * 4 + s * 4 + s * 4
+    wk.kernel = "segreduce_tile_f<256x16, float, plus>"
+    wk.step = lambda i: m.segreduce(vals[i % copies], segs[i % copies], "plus", 0.0,
+                                    out=outs[i % copies])
+    wk.tiles = lambda i: m.segreduce(vals[i % copies], segs[i % copies], "plus", 0.0,
+                                     out=outs[i % copies], phases=2)
+
+    def check():
+        got = m.segreduce(vals[0], segs[0], "plus", 0.0, out=outs[0])
+        lens = torch.diff(torch.cat([segs[0].long(), torch.tensor([n], device="cuda")]))
+        want = torch.segment_reduce(vals[0].double(), "sum", lengths=lens, unsafe=True)
+        ok = torch.all((got.double() - want).abs() <= 1e-5 * want.abs() + 1e-30)
+        # and a slice against the CPU oracle itself
+        from oracle import oracle
+        k = 1 << 14
+        cnt = int(w["segments"][k])
+        ref = oracle.segreduce(w["values"][:cnt], w["segments"][:k], "plus", 0.0)
+        ok2 = np.all(np.abs(got[:k - 1].cpu().numpy() - ref[:k - 1]) <=
+                     1e-5 * np.abs(ref[:k - 1]))
+        return bool(ok) and bool(ok2)
+    wk.check = check
+
+    def cpu():
+        from oracle import oracle
+        return lambda: oracle.segreduce(w["values"], w["segments"], "plus", 0.0)
+    wk.cpu = cpu
+    return wk
+
+
+def make_c3(copies, expand=False):
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    w = workloads.config3()
+    n, s = w["count"], w["segments"].size
+    segs = [_dev(w["segments"]) for _ in range(copies)]
+    vals = [_dev(w["values"]) for _ in range(copies)]
+    outs = [torch.empty(n, dtype=torch.int32, device="cuda") for _ in range(copies)]
+    wk = Workload()
+    wk.dtype = "i32"
+    wk.items = n
+    if expand:
+        wk.key = "c3_interval_expand_i32"
+        wk.name = "interval_expand int32, 2^24 Zipf(1.2) segments, 2^28 items"
+        wk.bytes = s * 4 + s * 4 + n * 4
+        wk.kernel = "transform_lbs_f<256x16, expand>"
+        wk.step = lambda i: m.interval_expand(vals[i % copies], n, segs[i % copies],
+                                              out=outs[i % copies])
+        wk.tiles = lambda i: m.interval_expand(vals[i % copies], n, segs[i % copies],
+                                               out=outs[i % copies], phases=2)
+    else:
+        wk.key = "c3_load_balance_search"
+        wk.name = "load_balance_search, 2^24 Zipf(1.2) segments, 2^28 items"
+        wk.bytes = s * 4 + n * 4
+        wk.kernel = "transform_lbs_f<256x16, store seg>"
+        wk.step = lambda i: m.load_balance_search(n, segs[i % copies], out=outs[i % copies])
+        wk.tiles = lambda i: m.load_balance_search(n, segs[i % copies], out=outs[i % copies],
+                                                   phases=2)
+
+    def check():
+        got = wk.step(0)
+        torch.cuda.synchronize()
+        step = 1 << 26
+        for lo in range(0, n, step):
+            idx = torch.arange(lo, min(lo + step, n), dtype=torch.int32, device="cuda")
+            want = torch.searchsorted(segs[0], idx, right=True) - 1
+            if expand:
+                want = vals[0][want]
+                if not torch.equal(got[lo:lo + step], want):
+                    return False
+            elif not torch.equal(got[lo:lo + step].long(), want):
+                return False
+        return True
+    wk.check = check
+
+    def cpu():
+        from oracle import oracle
+        if expand:
+            return lambda: oracle.interval_expand(w["values"], n, w["segments"])
+        return lambda: oracle.load_balance_search(n, w["segments"])
+    wk.cpu = cpu
+    return wk
+
+
+def make_c4(copies):
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    w = workloads.config4()
+    nnz, rows = w["nnz"], w["segments"].size
+    mats = [_dev(w["matrix"]) for _ in range(copies)]
+    cols = [_dev(w["columns"]) for _ in range(copies)]
+    segs = [_dev(w["segments"]) for _ in range(copies)]
+    x = _dev(w["vector"])
+    outs = [torch.empty(rows, dtype=torch.float32, device="cuda") for _ in range(copies)]
+    wk = Workload()
+    wk.key = "c4_spmv_f32"
+    wk.name = "spmv fp32, 2^22 rows, Zipf(1.5) row lengths (mean 16), %d nonzeros" % nnz
+    wk.dtype = "f32"
+    wk.items = nnz
+    wk.bytes = nnz * 8 + rows * 4 + rows * 4 + rows * 4
+    wk.kernel = "segreduce_tile_f<256x16, spmv float>"
+    wk.step = lambda i: m.spmv(mats[i % copies], cols[i % copies], x, segs[i % copies],
+                               out=outs[i % copies])
+    wk.tiles = lambda i: m.spmv(mats[i % copies], cols[i % copies], x, segs[i % copies],
+                                out=outs[i % copies], phases=2)
+
+    def check():
+        got = wk.step(0)
+        lens = torch.diff(torch.cat([segs[0].long(), torch.tensor([nnz], device="cuda")]))
+        prod = mats[0].double() * x.double()[cols[0].long()]
+        want = torch.segment_reduce(prod, "sum", lengths=lens, unsafe=True)
+        norm = torch.segment_reduce(prod.abs(), "sum", lengths=lens, unsafe=True)
+        return bool(torch.all((got.double() - want).abs() <= 1e-5 * norm + 1e-30))
+    wk.check = check
+
+    def cpu():
+        from oracle import oracle
+        return lambda: oracle.spmv(w["matrix"], w["columns"], w["vector"], w["segments"])
+    wk.cpu = cpu
+    return wk
+
+
+def make_c5(copies, kind):
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    w = workloads.config5(kind=kind)
+    n, s = w["values"].size, w["segments"].size
+    vals = [_dev(w["values"]) for _ in range(copies)]
+    segs = [_dev(w["segments"]) for _ in range(copies)]
+    outs = [torch.empty(s, dtype=vals[0].dtype, device="cuda") for _ in range(copies)]
+    wk = Workload()
+    wk.key = "c5_" + kind
+    wk.name = "segreduce %s, 2^27 values, 2^18 segments, four of ~2^25 items" % kind
+    wk.dtype = "f64" if kind == "f64max" else "i64"
+    wk.items = n
+    wk.bytes = n * 8 + s * 4 + s * 8
+    wk.kernel = "segreduce_tile_f<256x8, %s>" % kind
+    wk.step = lambda i: m.segreduce(vals[i % copies], segs[i % copies], w["op"], w["init"],
+                                    out=outs[i % copies])
+    wk.tiles = lambda i: m.segreduce(vals[i % copies], segs[i % copies], w["op"], w["init"],
+                                     out=outs[i % copies], phases=2)
+
+    def check():
+        got = wk.step(0)
+        lens = torch.diff(torch.cat([segs[0].long(), torch.tensor([n], device="cuda")]))
+        red = "max" if kind == "f64max" else "sum"
+        want = torch.segment_reduce(vals[0], red, lengths=lens, unsafe=True)
+        nz = lens > 0
+        return bool(torch.equal(got[nz], want[nz]))
+    wk.check = check
+
+    def cpu():
+        from oracle import oracle
+        return lambda: oracle.segreduce(w["values"], w["segments"], w["op"], w["init"])
+    wk.cpu = cpu
+    return wk
+
+
+def make_c1(copies):
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    from oracle import oracle
+    w = workloads.config1()
+    n, s = w["values"].size, w["segments"].size
+    vals, segs = _dev(w["values"]), _dev(w["segments"])
+    out = torch.empty(s, dtype=torch.int32, device="cuda")
+    wk = Workload()
+    wk.key = "c1_segreduce_i32"
+    wk.name = "segreduce int32 plus, 10^6 values, 10^4 segments"
+    wk.dtype = "i32"
+    wk.items = n
+    wk.bytes = n * 4 + s * 4 + s * 4
+    wk.kernel = "segreduce_tile_f<256x16, int, plus>"
+    wk.step = lambda i: m.segreduce(vals, segs, "plus", 0, out=out)
+    wk.tiles = lambda i: m.segreduce(vals, segs, "plus", 0, out=out, phases=2)
+    wk.check = lambda: bool(np.array_equal(
+        wk.step(0).cpu().numpy(), oracle.segreduce(w["values"], w["segments"], "plus", 0)))
+    wk.cpu = lambda: (lambda: oracle.segreduce(w["values"], w["segments"], "plus", 0))
+    return wk
+
+
+FACTORIES = {
+    "c1_segreduce_i32": make_c1,
+    "c2_segreduce_f32": make_c2,
+    "c3_load_balance_search": lambda c: make_c3(c, False),
+    "c3_interval_expand_i32": lambda c: make_c3(c, True),
+    "c4_spmv_f32": make_c4,
+    "c5_f64max": lambda c: make_c5(c, "f64max"),
+    "c5_i64sum": lambda c: make_c5(c, "i64sum"),
+}
+
+# HBM traffic of the dominant kernel per launch, from rocprofv3 --pmc
+# FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by what the same counters
+# read for a plain copy of known size.  None until measured.
+TRAFFIC_BYTES = {}
+
+
+def time_steps(fn, steps, warmup):
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(steps):
+        fn(warmup + i)
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) / steps
+
+
+def time_kernel_events(fn, steps, warmup):
+    """Average duration of one launch of the dominant kernel, from HIP events
+    recorded on the stream the kernels run on (torch's current stream)."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    total = 0.0
+    for i in range(steps):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn(warmup + i)
+        e1.record()
+        e1.synchronize()
+        total += e0.elapsed_time(e1)
+    return total / steps / 1e3
+
+
+def cpu_baseline(wk, budget_s=4.0):
+    run = wk.cpu()
+    reps, t_total = 0, 0.0
+    while reps < 1 or (t_total < budget_s and reps < 50):
+        t0 = time.perf_counter()
+        run()
+        t_total += time.perf_counter() - t0
+        reps += 1
+    sec = t_total / reps
+    return {"value": wk.bytes / sec / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "items_per_s": wk.items / sec,
+            "sample": "full workload, %d repetition(s), single thread, gcc -O3 -march=native "
+                      "(host has %d logical cores)" % (reps, os.cpu_count() or 0)}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=30)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="c2_segreduce_f32", choices=sorted(FACTORIES))
+    ap.add_argument("--copies", type=int, default=4)
+    ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--extra", default="c3_load_balance_search",
+                    help="comma-separated further workloads reported under 'others'")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: every box of this build has one, and the "
+                 "path under test uses no collective. Run with --gpus 1.")
+
+    import torch
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+
+    def measure(key, with_cpu):
+        wk = FACTORIES[key](args.copies)
+        if not wk.check():
+            sys.exit("parity check failed for %s: no throughput reported" % key)
+        sec = time_steps(wk.step, args.steps, args.warmup)
+        ksec = time_kernel_events(wk.tiles, args.steps, args.warmup)
+        res = {
+            "workload": key, "description": wk.name, "dtype": wk.dtype,
+            "ms_per_step": sec * 1e3, "GBps": wk.bytes / sec / 1e9,
+            "items_per_s": wk.items / sec,
+            "pct_hbm_peak": 100.0 * wk.bytes / sec / 1e9 / HBM_PEAK_GBPS,
+            "algorithmic_bytes": wk.bytes,
+            "roofline": {
+                "bound": "hbm", "kernel": wk.kernel,
+                "achieved": wk.bytes / ksec / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                "frac": wk.bytes / ksec / 1e9 / HBM_PEAK_GBPS,
+                "kernel_ms": ksec * 1e3,
+                "traffic": TRAFFIC_BYTES.get(key),
+            },
+        }
+        if with_cpu:
+            res["cpu_baseline"] = cpu_baseline(wk)
+        del wk
+        torch.cuda.empty_cache()
+        return res
+
+    main_res = measure(args.workload, not args.no_cpu)
+    others = {}
+    for key in [k for k in args.extra.split(",") if k and k != args.workload]:
+        r = measure(key, False)
+        others[key] = {k: r[k] for k in ("ms_per_step", "GBps", "items_per_s", "pct_hbm_peak")}
+        others[key]["roofline_frac"] = r["roofline"]["frac"]
+
+    line = {
+        "metric": "segreduce_input_GBps", "value": main_res["GBps"], "unit": "GB/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
+        "data": "synthetic (seeded numpy PCG64, seed 42), inputs resident in HBM, "
+                "%d rotating copies" % args.copies,
+        "config": {"workload": main_res["workload"], "description": main_res["description"],
+                   "algorithmic_bytes": main_res["algorithmic_bytes"]},
+        "items_per_s": main_res["items_per_s"], "pct_hbm_peak": main_res["pct_hbm_peak"],
+        "roofline": main_res["roofline"],
+    }
+    if "cpu_baseline" in main_res:
+        line["cpu_baseline"] = main_res["cpu_baseline"]
+    if others:
+        line["others"] = others
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

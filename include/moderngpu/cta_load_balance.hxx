@@ -68,12 +68,22 @@ struct chunk_width_t {
   };
 };
 
+// A tile's ranges are sized by the partition array.  If the caller's
+// segment starts are not ascending the splits can be inconsistent; force the
+// counts into [0, nv] so that no LDS or global access leaves its array (the
+// results are then meaningless, but nothing faults).
+MGPU_DEVICE inline merge_range_t clamp_tile_range(merge_range_t r, int nv) {
+  r.a_end = min(max(r.a_end, r.a_begin), r.a_begin + nv);
+  r.b_end = min(max(r.b_end, r.b_begin), r.b_begin + nv - (r.a_end - r.a_begin));
+  return r;
+}
+
 // Read W consecutive LDS elements starting at an index that is a multiple
 // of W.
 template<int W, typename type_t>
 MGPU_DEVICE inline void lds_load_chunk(const type_t* p, type_t (&x)[W]) {
-  if(W > 1) {
-    typedef typename vec_t<type_t, (W > 1 ? W : 2)>::type v_t;
+  if constexpr(W > 1) {
+    typedef typename vec_t<type_t, W>::type v_t;
     v_t v = *(const v_t*)p;
     PRAGMA_UNROLL
     for(int e = 0; e < W; ++e) x[e] = v[e];
@@ -82,8 +92,8 @@ MGPU_DEVICE inline void lds_load_chunk(const type_t* p, type_t (&x)[W]) {
 }
 template<int W, typename type_t>
 MGPU_DEVICE inline void lds_store_chunk(type_t* p, const type_t (&x)[W]) {
-  if(W > 1) {
-    typedef typename vec_t<type_t, (W > 1 ? W : 2)>::type v_t;
+  if constexpr(W > 1) {
+    typedef typename vec_t<type_t, W>::type v_t;
     v_t v;
     PRAGMA_UNROLL
     for(int e = 0; e < W; ++e) v[e] = x[e];
@@ -145,8 +155,9 @@ struct cta_load_balance_t {
     int num_segments, int tid, int cta, partition_it partitions,
     storage_t& storage) const {
 
-    merge_range_t range = compute_merge_range(count, num_segments, cta, nv,
-      partitions[cta], partitions[cta + 1]);
+    merge_range_t range = detail::clamp_tile_range(
+      compute_merge_range(count, num_segments, cta, nv,
+        partitions[cta], partitions[cta + 1]), nv);
     int a_count = range.a_count();
     int b_count = range.b_count();
     int* slots = storage.indices;
@@ -281,7 +292,7 @@ struct cached_segment_load_t {
       __syncthreads();
     } else {
       strided_iterate<nt, vt, vt0>([&](int i, int) {
-        loaded[i] = mgpu::load(iterators, segments[i]);
+        loaded[i] = mgpu::load(iterators, max(segments[i], 0));
       }, tid, count);
     }
     return loaded;

@@ -60,8 +60,8 @@ template<typename type_t, int W>
 struct pointer_loader_t {
   MGPU_DEVICE static void load(const type_t* input, int index,
     type_t (&x)[W]) {
-    if(W > 1) {
-      typedef typename vec_t<type_t, (W > 1 ? W : 2)>::type_u v_t;
+    if constexpr(W > 1) {
+      typedef typename vec_t<type_t, W>::type_u v_t;
       v_t v = *(const v_t*)(input + index);
       PRAGMA_UNROLL
       for(int e = 0; e < W; ++e) x[e] = v[e];
@@ -94,8 +94,8 @@ struct tile_loader_t<spmv_input_t<type_t>, type_t, W> {
     int c[W];
     pointer_loader_t<type_t, W>::load(in.matrix, index, a);
     // Columns are 4-byte: W of them are 16 bytes or less.
-    if(W > 1) {
-      typedef typename vec_t<int, (W > 1 ? W : 2)>::type_u v_t;
+    if constexpr(W > 1) {
+      typedef typename vec_t<int, W>::type_u v_t;
       v_t v = *(const v_t*)(in.columns + index);
       PRAGMA_UNROLL
       for(int e = 0; e < W; ++e) c[e] = v[e];
@@ -153,8 +153,9 @@ struct segreduce_tile_f {
       typename segscan_t::storage_t segscan;
     } shared;
 
-    merge_range_t range = compute_merge_range(count, num_segments, cta, nv,
-      mp_data[cta], mp_data[cta + 1]);
+    merge_range_t range = clamp_tile_range(
+      compute_merge_range(count, num_segments, cta, nv,
+        mp_data[cta], mp_data[cta + 1]), nv);
     int a_count = range.a_count();
     int b_count = range.b_count();
 

@@ -1,0 +1,223 @@
+// Test-only kernels that expose the CTA-level primitives (cta_scan_t,
+// cta_reduce_t, cta_segscan_t, the wave-level helpers) through a small C ABI
+// so the Python tests can compare them with serial host scans.
+// Built into tests/csrc/libmgpu_test_kernels.so; not part of the product.
+#include <moderngpu/cta_reduce.hxx>
+#include <moderngpu/cta_scan.hxx>
+#include <moderngpu/cta_segscan.hxx>
+#include <moderngpu/transform.hxx>
+
+using namespace mgpu;
+
+namespace {
+
+class bare_context_t : public context_t {
+  hipDeviceProp_t _props;
+public:
+  bare_context_t() { memset(&_props, 0, sizeof(_props)); }
+  virtual const hipDeviceProp_t& props() const { return _props; }
+  virtual int ptx_version() const { return arch_version_gfx950; }
+  virtual hipStream_t stream() { return 0; }
+  virtual void* alloc(size_t, memory_space_t) { return nullptr; }
+  virtual void free(void*, memory_space_t) { }
+  virtual void synchronize() { }
+  virtual hipEvent_t event() { return nullptr; }
+  virtual void timer_begin() { }
+  virtual double timer_end() { return 0; }
+};
+
+template<typename type_t>
+struct op_any_t {
+  int op;   // 0 plus, 1 max, 2 min, 3 "left then right" non-commutative
+  MGPU_DEVICE type_t operator()(type_t a, type_t b) const {
+    switch(op) {
+      case 0: return a + b;
+      case 1: return mgpu::max(a, b);
+      case 2: return mgpu::min(a, b);
+      default: return (type_t)(a * (type_t)3 + b);   // order-sensitive
+    }
+  }
+};
+
+template<int nt, typename type_t>
+void run_scan(const type_t* in, int count, type_t* out, type_t* red, int op,
+  type_t init, int inclusive) {
+  bare_context_t context;
+  cta_launch<nt>([=]MGPU_DEVICE(int tid, int) {
+    typedef cta_scan_t<nt, type_t> scan_t;
+    __shared__ typename scan_t::storage_t storage;
+    scan_result_t<type_t> r = scan_t().scan(tid, in[tid], storage, count,
+      op_any_t<type_t> { op }, init,
+      inclusive ? scan_type_inc : scan_type_exc);
+    out[tid] = r.scan;
+    if(!tid) *red = r.reduction;
+  }, 1, context);
+}
+
+template<int nt, int vt, typename type_t>
+void run_scan_vt(const type_t* in, int count, type_t* out, type_t* red,
+  int op, type_t init, int inclusive, type_t carry_in, int use_carry) {
+  bare_context_t context;
+  cta_launch<nt>([=]MGPU_DEVICE(int tid, int) {
+    typedef cta_scan_t<nt, type_t> scan_t;
+    __shared__ typename scan_t::storage_t storage;
+    array_t<type_t, vt> x;
+    iterate<vt>([&](int i) { x[i] = in[vt * tid + i]; });
+    scan_result_t<type_t, vt> r = scan_t().template scan<vt>(tid, x, storage,
+      carry_in, 0 != use_carry, count, op_any_t<type_t> { op }, init,
+      inclusive ? scan_type_inc : scan_type_exc);
+    iterate<vt>([&](int i) { out[vt * tid + i] = r.scan[i]; });
+    if(!tid) *red = r.reduction;
+  }, 1, context);
+}
+
+template<int nt, typename type_t>
+void run_reduce(const type_t* in, int count, type_t* out, int op,
+  int all_return) {
+  bare_context_t context;
+  cta_launch<nt>([=]MGPU_DEVICE(int tid, int) {
+    typedef cta_reduce_t<nt, type_t> reduce_t;
+    __shared__ typename reduce_t::storage_t storage;
+    type_t r = reduce_t().reduce(tid, in[tid], storage, count,
+      op_any_t<type_t> { op }, 0 != all_return);
+    out[tid] = r;
+  }, 1, context);
+}
+
+template<int nt, typename type_t>
+void run_segscan(const type_t* in, const int* heads, const int* carries,
+  type_t* scan_out, int* carry_in_out, int* left_out, int* has_left_out,
+  type_t* red, int op, type_t init) {
+  bare_context_t context;
+  cta_launch<nt>([=]MGPU_DEVICE(int tid, int) {
+    typedef cta_segscan_t<nt, type_t> segscan_t;
+    __shared__ typename segscan_t::storage_t storage;
+    segscan_result_t<type_t> r = segscan_t().segscan(tid, 0 != heads[tid],
+      0 != carries[tid], in[tid], storage, init, op_any_t<type_t> { op });
+    scan_out[tid] = r.scan;
+    carry_in_out[tid] = r.has_carry_in;
+    left_out[tid] = r.left_lane;
+    has_left_out[tid] = r.has_left_head;
+    if(!tid) *red = r.reduction;
+  }, 1, context);
+}
+
+template<int nt>
+void run_scan_bool(const int* in, int* out, int* red) {
+  bare_context_t context;
+  cta_launch<nt>([=]MGPU_DEVICE(int tid, int) {
+    typedef cta_scan_t<nt, bool> scan_t;
+    __shared__ typename scan_t::storage_t storage;
+    scan_result_t<int> r = scan_t().scan(tid, 0 != in[tid], storage);
+    out[tid] = r.scan;
+    if(!tid) *red = r.reduction;
+  }, 1, context);
+}
+
+// shfl_up / shfl_down / shfl_up_op / shfl_down_op / wave_allreduce on one
+// wavefront.  mode selects the function.
+void run_shfl(const int* in, int* out, int mode, int offset, int width) {
+  bare_context_t context;
+  cta_launch<64>([=]MGPU_DEVICE(int tid, int) {
+    int x = in[tid];
+    int y = 0;
+    switch(mode) {
+      case 0: y = shfl_up(x, offset, width); break;
+      case 1: y = shfl_down(x, offset, width); break;
+      case 2: y = shfl_up_op(x, offset, plus_t<int>(), width); break;
+      case 3: y = shfl_down_op(x, offset, plus_t<int>(), width); break;
+      case 4: y = wave_allreduce(x, op_any_t<int> { 3 }, tid); break;
+      case 5: y = lane_id(); break;
+      case 6: y = (int)popc(ballot(x & 1)); break;
+    }
+    out[tid] = y;
+  }, 1, context);
+}
+
+#define BY_NT(fn, ...)                                                        \
+  switch(nt) {                                                                \
+    case 64: fn<64>(__VA_ARGS__); break;                                      \
+    case 128: fn<128>(__VA_ARGS__); break;                                    \
+    case 256: fn<256>(__VA_ARGS__); break;                                    \
+    case 512: fn<512>(__VA_ARGS__); break;                                    \
+    case 1024: fn<1024>(__VA_ARGS__); break;                                  \
+    default: return -1;                                                       \
+  }
+
+#define BY_NT_T(fn, T, ...)                                                   \
+  switch(nt) {                                                                \
+    case 64: fn<64, T>(__VA_ARGS__); break;                                   \
+    case 128: fn<128, T>(__VA_ARGS__); break;                                 \
+    case 256: fn<256, T>(__VA_ARGS__); break;                                 \
+    case 512: fn<512, T>(__VA_ARGS__); break;                                 \
+    case 1024: fn<1024, T>(__VA_ARGS__); break;                               \
+    default: return -1;                                                       \
+  }
+
+int finish() {
+  hipError_t e = hipDeviceSynchronize();
+  return (int)(e != hipSuccess ? e : hipGetLastError());
+}
+
+} // namespace
+
+#define API extern "C" __attribute__((visibility("default")))
+
+API int tk_scan_i32(int nt, const int* in, int count, int* out, int* red,
+  int op, int init, int inclusive) {
+  BY_NT_T(run_scan, int, in, count, out, red, op, init, inclusive)
+  return finish();
+}
+API int tk_scan_i64(int nt, const long long* in, int count, long long* out,
+  long long* red, int op, long long init, int inclusive) {
+  BY_NT_T(run_scan, long long, in, count, out, red, op, init, inclusive)
+  return finish();
+}
+API int tk_scan_f64(int nt, const double* in, int count, double* out,
+  double* red, int op, double init, int inclusive) {
+  BY_NT_T(run_scan, double, in, count, out, red, op, init, inclusive)
+  return finish();
+}
+API int tk_scan_vt_i32(int nt, int vt, const int* in, int count, int* out,
+  int* red, int op, int init, int inclusive, int carry_in, int use_carry) {
+  if(nt == 128 && vt == 7)
+    run_scan_vt<128, 7, int>(in, count, out, red, op, init, inclusive, carry_in, use_carry);
+  else if(nt == 256 && vt == 4)
+    run_scan_vt<256, 4, int>(in, count, out, red, op, init, inclusive, carry_in, use_carry);
+  else if(nt == 64 && vt == 3)
+    run_scan_vt<64, 3, int>(in, count, out, red, op, init, inclusive, carry_in, use_carry);
+  else return -1;
+  return finish();
+}
+API int tk_reduce_i32(int nt, const int* in, int count, int* out, int op,
+  int all_return) {
+  BY_NT_T(run_reduce, int, in, count, out, op, all_return)
+  return finish();
+}
+API int tk_reduce_f64(int nt, const double* in, int count, double* out,
+  int op, int all_return) {
+  BY_NT_T(run_reduce, double, in, count, out, op, all_return)
+  return finish();
+}
+API int tk_segscan_i32(int nt, const int* in, const int* heads,
+  const int* carries, int* scan_out, int* carry_in_out, int* left_out,
+  int* has_left_out, int* red, int op, int init) {
+  BY_NT_T(run_segscan, int, in, heads, carries, scan_out, carry_in_out,
+    left_out, has_left_out, red, op, init)
+  return finish();
+}
+API int tk_segscan_i64(int nt, const long long* in, const int* heads,
+  const int* carries, long long* scan_out, int* carry_in_out, int* left_out,
+  int* has_left_out, long long* red, int op, long long init) {
+  BY_NT_T(run_segscan, long long, in, heads, carries, scan_out, carry_in_out,
+    left_out, has_left_out, red, op, init)
+  return finish();
+}
+API int tk_scan_bool(int nt, const int* in, int* out, int* red) {
+  BY_NT(run_scan_bool, in, out, red)
+  return finish();
+}
+API int tk_shfl(const int* in, int* out, int mode, int offset, int width) {
+  run_shfl(in, out, mode, offset, width);
+  return finish();
+}

@@ -1,0 +1,35 @@
+"""Runs the C++ callers written against the mgpu:: template API (same shape as
+the reference's tests/test_segreduce.cu and tests/test_load_balance.cu, plus
+user functors, user types and custom launch boxes).  They are compiled in-tree
+by tests/csrc/Makefile and exit non-zero on any mismatch."""
+import os
+import subprocess
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
+
+
+def _run(name, *args):
+    path = os.path.join(BIN, name)
+    assert os.path.exists(path), "build tests/csrc first (make -C tests/csrc)"
+    proc = subprocess.run([path] + [str(a) for a in args], capture_output=True,
+                          text=True, timeout=110)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    return proc.stdout
+
+
+def test_reference_style_segreduce(dev):
+    out = _run("test_segreduce", 10_000_000, 100_000, 5)
+    assert "passed" in out
+    out = _run("test_segreduce", 1_000_000, 100, 3)     # many short segments
+    assert "passed" in out
+
+
+def test_reference_style_load_balance(dev):
+    assert "passed" in _run("test_load_balance")
+
+
+def test_template_paths(dev):
+    assert "all passed" in _run("test_templates")

@@ -1,0 +1,201 @@
+"""Segmented reduction through the C ABI against the CPU oracle: bit-exact for
+integer types and for max/min of floats; for floating sums within the stated
+tolerance of an exact (math.fsum / float64) sum and of the oracle's serial sum.
+
+Tolerances (relative to sum |x| of the segment; reassociation only):
+    float32 sums 1e-5, float64 sums 1e-12.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from util import lengths_of, random_segments, segment_layouts
+
+pytestmark = pytest.mark.gpu
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+TOL = {np.dtype(np.float32): 1e-5, np.dtype(np.float64): 1e-12}
+
+
+def _dev(a):
+    import torch
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _gpu_segreduce(values, segs, op, init):
+    import torch
+    import moderngpu_amd as m
+    unsigned = values.dtype in (np.uint32, np.uint64)
+    v = values.view(np.int32 if values.dtype == np.uint32 else np.int64) if unsigned else values
+    # Poison the output so segments nobody writes are noticed.
+    out = torch.full((segs.size,), 0x5a5a5a5a if v.dtype.kind in "iu" else float("nan"),
+                     dtype=_dev(v[:0]).dtype, device="cuda")
+    m.segreduce(_dev(v), _dev(segs), op, init, out=out, unsigned=unsigned)
+    got = out.cpu().numpy()
+    return got.view(values.dtype) if unsigned else got
+
+
+def _abs_sums(values, segs):
+    lens = lengths_of(segs, values.size)
+    out = np.zeros(segs.size)
+    nz = lens > 0
+    if nz.any() and values.size:
+        out[nz] = np.add.reduceat(np.abs(values.astype(np.float64)), segs[nz].astype(np.int64))
+    return out
+
+
+def _check(values, segs, op, init, oracle, name=""):
+    got = _gpu_segreduce(values, segs, op, init)
+    want = oracle.segreduce(values, segs, op, init)
+    if values.dtype.kind == "f" and op == "plus":
+        # "exact": extended-precision (x87 long double) sum of the same inputs.
+        lens = lengths_of(segs, values.size)
+        exact = np.zeros(segs.size, dtype=np.longdouble)
+        if values.size and (lens > 0).any():
+            exact[lens > 0] = np.add.reduceat(values.astype(np.longdouble),
+                                              segs[lens > 0].astype(np.int64))
+        bound = TOL[values.dtype] * _abs_sums(values, segs)
+        assert np.array_equal(got[lens == 0], want[lens == 0]), name
+        assert np.all(np.abs(got.astype(np.longdouble) - exact)[lens > 0] <= (bound + 1e-300)[lens > 0]), name
+        # and next to the oracle's serial sum in the same type
+        assert np.all(np.abs(got.astype(np.float64) - want.astype(np.float64)) <= 4 * bound + 1e-300), name
+    else:
+        assert got.tobytes() == want.tobytes(), (name, op, values.dtype)
+
+
+def test_golden_mod13(dev, oracle):
+    """The reference test's shape: transform_segreduce of index % 13, int32 +,
+    init -1, starts from std::mt19937 (tests/test_segreduce.cu:16-49)."""
+    import moderngpu_amd as m
+    g = json.load(open(os.path.join(GOLDEN, "segreduce_mod13.json")))
+    for c in g["cases"]:
+        segs = np.array(c["segments"], dtype=np.int32)
+        want = np.array(c["expected"], dtype=np.int32)
+        got = m.transform_segreduce_mod13(c["count"], _dev(segs), g["init"]).cpu().numpy()
+        assert np.array_equal(got, want), c["seed"]
+        vals = (np.arange(c["count"]) % 13).astype(np.int32)
+        assert np.array_equal(_gpu_segreduce(vals, segs, "plus", g["init"]), want)
+
+
+def test_mod13_large_closed_form(dev):
+    """The reference test's own size class: 10^7 items in 100 segments, so
+    every segment spans many tiles (exercises the carry spine)."""
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    count = 10_000_000
+    for seed in range(3):
+        segs = workloads.reference_test_segments(count, 100, seed)
+        got = m.transform_segreduce_mod13(count, _dev(segs), -1).cpu().numpy()
+
+        def prefix(n):
+            n = n.astype(np.int64)
+            r = n % 13
+            return 78 * (n // 13) + r * (r - 1) // 2
+        ends = np.append(segs[1:], count)
+        want = np.where(ends > segs, prefix(ends) - prefix(segs), -1).astype(np.int32)
+        assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("dtype", [np.int32, np.uint32, np.int64, np.uint64,
+                                   np.float32, np.float64])
+@pytest.mark.parametrize("op", ["plus", "maximum", "minimum"])
+def test_layouts_all_types(dev, oracle, dtype, op):
+    import moderngpu_amd as m
+    rng = np.random.default_rng(21)
+    code = {np.int32: 0, np.uint32: 1, np.int64: 2, np.uint64: 3,
+            np.float32: 4, np.float64: 5}[dtype]
+    nv = m.segreduce_tile_size(code)
+    for name, count, segs in segment_layouts(rng, nv):
+        if np.dtype(dtype).kind == "f":
+            values = (rng.standard_normal(count) * 100).astype(dtype)
+            init = dtype(-7.5)
+        else:
+            info = np.iinfo(dtype)
+            values = rng.integers(info.min, info.max, size=count, dtype=dtype, endpoint=True)
+            init = 42
+        _check(values, segs, op, init, oracle, name)
+
+
+def test_float_specials(dev, oracle):
+    # +0/-0 ties and infinities through max/min must match the host loop's
+    # left-operand-wins rule bit for bit.
+    rng = np.random.default_rng(22)
+    count = 20000
+    segs = random_segments(rng, count, 700)
+    for dtype in (np.float32, np.float64):
+        pool = np.array([0.0, -0.0, 1.0, -1.0, np.inf, -np.inf, 3.5], dtype=dtype)
+        values = pool[rng.integers(0, pool.size, size=count)]
+        for op in ("maximum", "minimum"):
+            _check(values, segs, op, dtype(2.0), oracle, "specials")
+
+
+def test_config1(dev, oracle):
+    from moderngpu_amd import workloads
+    w = workloads.config1()
+    _check(w["values"], w["segments"], "plus", 0, oracle, "config1")
+    # the reference test's closed upper bound: a start may equal count
+    segs = workloads.reference_test_segments(w["values"].size, 10000, 42)
+    _check(w["values"], segs, "plus", -1, oracle, "config1_closed")
+
+
+def test_config2_scaled(dev, oracle):
+    from moderngpu_amd import workloads
+    w = workloads.config2(scale=8)
+    _check(w["values"], w["segments"], "plus", 0.0, oracle, "config2/8")
+
+
+@pytest.mark.parametrize("kind", ["f64max", "i64sum"])
+def test_config5_scaled(dev, oracle, kind):
+    from moderngpu_amd import workloads
+    w = workloads.config5(scale=8, kind=kind)
+    _check(w["values"], w["segments"], w["op"], w["init"], oracle, "config5/8")
+
+
+def test_spine_levels(dev, oracle):
+    """More than 1024 tiles in one segment forces the second spine level; a
+    segment that begins exactly on a tile edge takes the overwrite path."""
+    import moderngpu_amd as m
+    rng = np.random.default_rng(23)
+    nv = m.segreduce_tile_size(0)
+    count = 2600 * nv + 123
+    values = rng.integers(-1000, 1000, size=count).astype(np.int32)
+    for segs in ([0], [0, 5], [0, nv - 1], [0, nv - 1, 1030 * nv - 1030, 2000 * nv],
+                 [0, 0, 0, count - 1, count, count]):
+        _check(values, np.array(segs, dtype=np.int32), "plus", -3, oracle, str(segs))
+        _check(values, np.array(segs, dtype=np.int32), "maximum", -3, oracle, str(segs))
+
+
+def test_full_size_config2_properties(dev):
+    """2^26 fp32 items: compared on the device with torch.segment_reduce
+    (independent code) in float64, tolerance 1e-5 * sum|x|."""
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    w = workloads.config2()
+    values, segs = _dev(w["values"]), _dev(w["segments"])
+    got = m.segreduce(values, segs, "plus", 0.0)
+    lens = torch.diff(torch.cat([segs.long(), torch.tensor([values.numel()], device=dev)]))
+    want = torch.segment_reduce(values.double(), "sum", lengths=lens, unsafe=True)
+    assert torch.all((got.double() - want).abs() <= 1e-5 * want.abs() + 1e-30)
+    assert torch.all(got[lens == 0] == 0)
+
+
+@pytest.mark.parametrize("kind", ["f64max", "i64sum"])
+def test_full_size_config5_properties(dev, kind):
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    w = workloads.config5(kind=kind)
+    values, segs = _dev(w["values"]), _dev(w["segments"])
+    got = m.segreduce(values, segs, w["op"], w["init"])
+    lens = torch.diff(torch.cat([segs.long(), torch.tensor([values.numel()], device=dev)]))
+    if kind == "i64sum":
+        want = torch.segment_reduce(values, "sum", lengths=lens, unsafe=True)
+        assert torch.equal(got, want)
+        assert int(got.sum().item()) == int(values.sum().item())
+    else:
+        want = torch.segment_reduce(values, "max", lengths=lens, unsafe=True)
+        nz = lens > 0
+        assert torch.equal(got[nz], want[nz])
+        assert torch.all(torch.isinf(got[~nz]) & (got[~nz] < 0))
