@@ -198,9 +198,13 @@ def make_c5(copies, kind):
     def check():
         got = wk.step(0)
         lens = torch.diff(torch.cat([segs[0].long(), torch.tensor([n], device="cuda")]))
-        red = "max" if kind == "f64max" else "sum"
-        want = torch.segment_reduce(vals[0], red, lengths=lens, unsafe=True)
         nz = lens > 0
+        if kind == "f64max":
+            want = torch.segment_reduce(vals[0], "max", lengths=lens, unsafe=True)
+        else:       # wrapping prefix sums (torch has no int64 segment_reduce)
+            prefix = torch.cat([torch.zeros(1, dtype=torch.int64, device="cuda"),
+                                torch.cumsum(vals[0], 0)])
+            want = prefix[segs[0].long() + lens] - prefix[segs[0].long()]
         return bool(torch.equal(got[nz], want[nz]))
     wk.check = check
 

@@ -237,7 +237,9 @@ struct segreduce_tile_f {
     auto fold_to = [&](int p, int e) -> type_t {
       int te = e / vt;
       type_t v = shared.values[layout_t::index(e)];
-      if(p < te * vt) v = op(shared.flow[te], v);
+      // thread 0 has nothing flowing in; p may be negative for the segment
+      // that was open when the tile began.
+      if(te && p < te * vt) v = op(shared.flow[te], v);
       return v;
     };
 

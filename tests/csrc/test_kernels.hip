@@ -28,13 +28,14 @@ public:
 
 template<typename type_t>
 struct op_any_t {
-  int op;   // 0 plus, 1 max, 2 min, 3 "left then right" non-commutative
+  int op;   // 0 plus, 1 max, 2 min, 3 left projection (associative, not
+            // commutative: exposes swapped operands)
   MGPU_DEVICE type_t operator()(type_t a, type_t b) const {
     switch(op) {
       case 0: return a + b;
       case 1: return mgpu::max(a, b);
       case 2: return mgpu::min(a, b);
-      default: return (type_t)(a * (type_t)3 + b);   // order-sensitive
+      default: return a;
     }
   }
 };
