@@ -268,22 +268,22 @@ def time_steps(fn, steps, warmup):
 
 
 def time_kernel_events(fn, steps, warmup):
-    """Average duration of one launch of the dominant kernel, from HIP events
-    recorded on the stream the kernels run on (torch's current stream)."""
+    """Average duration of one launch of the dominant kernel: `steps` launches
+    queued back to back between two HIP events recorded on the stream the
+    kernels run on (torch's current stream), so the figure is device time per
+    launch, not host launch latency."""
     import torch
     for i in range(warmup):
         fn(i)
     torch.cuda.synchronize()
-    total = 0.0
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
     for i in range(steps):
-        e0 = torch.cuda.Event(enable_timing=True)
-        e1 = torch.cuda.Event(enable_timing=True)
-        e0.record()
         fn(warmup + i)
-        e1.record()
-        e1.synchronize()
-        total += e0.elapsed_time(e1)
-    return total / steps / 1e3
+    e1.record()
+    e1.synchronize()
+    return e0.elapsed_time(e1) / steps / 1e3
 
 
 def cpu_baseline(wk, budget_s=4.0):

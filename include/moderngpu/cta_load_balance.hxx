@@ -45,11 +45,15 @@ struct vec_t {
 };
 
 // Tile element p lives at LDS element index(p).  W = elements per 16-byte
-// chunk (1 disables chunking and padding).
+// chunk (1 disables chunking and padding).  One spare chunk follows every
+// MGPU_TILE_PAD_CHUNKS chunks.
+#ifndef MGPU_TILE_PAD_CHUNKS
+#define MGPU_TILE_PAD_CHUNKS 8
+#endif
 template<int W>
 struct tile_layout_t {
   MGPU_HOST_DEVICE static constexpr int index(int p) {
-    return W > 1 ? p + (p / (8 * W)) * W : p;
+    return W > 1 ? p + (p / (MGPU_TILE_PAD_CHUNKS * W)) * W : p;
   }
   MGPU_HOST_DEVICE static constexpr int capacity(int n) {
     return index(n) + 2 * W;
@@ -68,13 +72,22 @@ struct chunk_width_t {
   };
 };
 
-// A tile's ranges are sized by the partition array.  If the caller's
-// segment starts are not ascending the splits can be inconsistent; force the
-// counts into [0, nv] so that no LDS or global access leaves its array (the
-// results are then meaningless, but nothing faults).
-MGPU_DEVICE inline merge_range_t clamp_tile_range(merge_range_t r, int nv) {
-  r.a_end = min(max(r.a_end, r.a_begin), r.a_begin + nv);
-  r.b_end = min(max(r.b_end, r.b_begin), r.b_begin + nv - (r.a_end - r.a_begin));
+// The tile's item and segment ranges from the two splits at its ends, forced
+// to be consistent: each split inside what its cross-diagonal allows, ends not
+// before begins, at most nv elements.  For well-formed input (ascending
+// starts) this changes nothing; for malformed input it keeps every LDS and
+// global access of the tile kernels inside its array (results are then
+// meaningless, but nothing faults).
+MGPU_DEVICE inline merge_range_t tile_range(int count, int num_segments,
+  int cta, int nv, int mp0, int mp1) {
+  int total = count + num_segments;
+  int diag0 = nv * cta;
+  int diag1 = min(total, diag0 + nv);
+  mp0 = min(max(mp0, max(0, diag0 - num_segments)), min(diag0, count));
+  mp1 = min(max(mp1, max(0, diag1 - num_segments)), min(diag1, count));
+  mp1 = min(max(mp1, mp0), mp0 + nv);
+  merge_range_t r { mp0, mp1, diag0 - mp0, diag1 - mp1 };
+  r.b_end = min(max(r.b_end, r.b_begin), r.b_begin + nv - (mp1 - mp0));
   return r;
 }
 
@@ -155,9 +168,8 @@ struct cta_load_balance_t {
     int num_segments, int tid, int cta, partition_it partitions,
     storage_t& storage) const {
 
-    merge_range_t range = detail::clamp_tile_range(
-      compute_merge_range(count, num_segments, cta, nv,
-        partitions[cta], partitions[cta + 1]), nv);
+    merge_range_t range = detail::tile_range(count, num_segments, cta, nv,
+      partitions[cta], partitions[cta + 1]);
     int a_count = range.a_count();
     int b_count = range.b_count();
     int* slots = storage.indices;

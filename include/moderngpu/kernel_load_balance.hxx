@@ -76,9 +76,8 @@ void transform_lbs_launch(func_t f, int count, segments_it segments,
 
   if(count + num_segments <= 0) return;
   if(phases & lbs_phase_partition)
-    merge_path_partitions_into<bounds_upper>(counting_iterator_t<int>(0),
-      (int64_t)count, segments, (int64_t)num_segments,
-      (int64_t)launch_t::nv(context), less_t<int>(), mp_data, context);
+    load_balance_partitions_into((int64_t)count, segments, num_segments,
+      launch_t::nv(context), mp_data, context);
 
   if(phases & lbs_phase_tiles) {
     transform_lbs_f<launch_t, func_t, segments_it, pointers_t, int>

@@ -26,16 +26,16 @@
 //       The segment that was already open when the tile began is reported as
 //       a (segment, partial) carry for the spine.
 //   K3  segreduce_spine_f folds the per-tile carries of segments that span
-//       tiles into output[]; 1024 carries per CTA, repeated on the per-CTA
-//       carries until one CTA is left.
+//       tiles into output[] in one launch (1024 carries per CTA; a run of
+//       carries that crosses CTAs is finished by the CTA it ends in).
 // The CUDA reference instead walks vt + 1 merged elements per thread through
-// dependent shared-memory reads and keeps an "overwrite" bit per tile; here
-// the spine decides between combine and overwrite by comparing the segment's
-// start with the first item of the tile that carried it.
+// dependent shared-memory reads and runs a recursive fix-up, one launch per
+// level.
 #pragma once
 #include "search.hxx"
 #include "cta_load_balance.hxx"
 #include "cta_segscan.hxx"
+#include "cta_reduce.hxx"
 #include "transform.hxx"
 #include "memory.hxx"
 
@@ -107,6 +107,78 @@ struct tile_loader_t<spmv_input_t<type_t>, type_t, W> {
 };
 
 ////////////////////////////////////////////////////////////////////////////////
+// One step of the thread-serial segmented scan: the running fold `prev`
+// continues into `cur` unless bit i of `bits` marks a segment start at this
+// item.  The generic form is a compare and a select around op().  For the
+// built-in operators on 4/8-byte arithmetic types the select folds into bit
+// arithmetic (no compare, no SGPR mask round trip):
+//   plus:     cur + (prev with all bits cleared when a segment starts here)
+//   max/min:  op(start ? cur : prev, cur), the choice done with one
+//             bitfield-insert per 32-bit word; op(cur, cur) == cur.
+// For floating-point plus a segment made only of -0.0 sums to +0.0; sums are
+// compared with a tolerance, and max/min stay bit-exact.
+
+template<typename op_t, typename type_t, typename enable_t = void>
+struct segscan_step_t {
+  MGPU_DEVICE static type_t step(type_t prev, type_t cur, unsigned bits,
+    int i, op_t op) {
+    return ((bits >> i) & 1) ? cur : op(prev, cur);
+  }
+};
+
+template<typename type_t>
+struct bitwise_word_t {
+  typedef typename std::conditional<sizeof(type_t) == 8, unsigned long long,
+    unsigned>::type type;
+  MGPU_DEVICE static type to(type_t x) {
+    type y; __builtin_memcpy(&y, &x, sizeof(y)); return y;
+  }
+  MGPU_DEVICE static type_t from(type y) {
+    type_t x; __builtin_memcpy(&x, &y, sizeof(x)); return x;
+  }
+  // All ones if bit i of bits is set, else zero.
+  MGPU_DEVICE static type spread(unsigned bits, int i) {
+    // the builtin's result is declared unsigned: make it signed before
+    // widening so that the 64-bit mask is all ones, not 32 ones.
+    return (type)(long long)(int)__builtin_amdgcn_sbfe(bits, i, 1);
+  }
+};
+
+template<typename type_t>
+struct is_word_arithmetic_t {
+  enum { value = std::is_arithmetic<type_t>::value &&
+    (sizeof(type_t) == 4 || sizeof(type_t) == 8) };
+};
+
+template<typename type_t>
+struct segscan_step_t<plus_t<type_t>, type_t,
+  enable_if_t<is_word_arithmetic_t<type_t>::value> > {
+  MGPU_DEVICE static type_t step(type_t prev, type_t cur, unsigned bits,
+    int i, plus_t<type_t>) {
+    typedef bitwise_word_t<type_t> w;
+    return w::from(w::to(prev) & ~w::spread(bits, i)) + cur;
+  }
+};
+
+template<typename op_t, typename type_t>
+struct segscan_select_step_t {
+  MGPU_DEVICE static type_t step(type_t prev, type_t cur, unsigned bits,
+    int i, op_t op) {
+    typedef bitwise_word_t<type_t> w;
+    typename w::type m = w::spread(bits, i);
+    return op(w::from((m & w::to(cur)) | (~m & w::to(prev))), cur);
+  }
+};
+template<typename type_t>
+struct segscan_step_t<maximum_t<type_t>, type_t,
+  enable_if_t<is_word_arithmetic_t<type_t>::value> > :
+  segscan_select_step_t<maximum_t<type_t>, type_t> { };
+template<typename type_t>
+struct segscan_step_t<minimum_t<type_t>, type_t,
+  enable_if_t<is_word_arithmetic_t<type_t>::value> > :
+  segscan_select_step_t<minimum_t<type_t>, type_t> { };
+
+////////////////////////////////////////////////////////////////////////////////
 // Default tiles on gfx950, by value size.
 
 template<typename type_t>
@@ -114,6 +186,23 @@ struct segreduce_launch_default_t {
   typedef launch_box_t<
     arch_gfx950_cta<256, (sizeof(type_t) > 4 ? 8 : 16)>
   > type_t_;
+};
+
+////////////////////////////////////////////////////////////////////////////////
+// What a tile (or a spine CTA) passes on: the segment its leading partial
+// belongs to, and whether output[segment] still has to be created ("fresh")
+// rather than combined with.  seg >= 0: combine; ~seg (negative): fresh;
+// none: nothing to pass on.
+
+struct carry_code_t {
+  enum : int { none = (int)0x80000000 };
+  MGPU_HOST_DEVICE static int make(int seg, bool fresh) {
+    return fresh ? ~seg : seg;
+  }
+  MGPU_HOST_DEVICE static int seg(int code) {      // -1 for none
+    return none == code ? -1 : (code < 0 ? ~code : code);
+  }
+  MGPU_HOST_DEVICE static bool fresh(int code) { return code < 0; }
 };
 
 ////////////////////////////////////////////////////////////////////////////////
@@ -153,13 +242,24 @@ struct segreduce_tile_f {
       typename segscan_t::storage_t segscan;
     } shared;
 
-    merge_range_t range = clamp_tile_range(
-      compute_merge_range(count, num_segments, cta, nv,
-        mp_data[cta], mp_data[cta + 1]), nv);
+    merge_range_t range = tile_range(count, num_segments, cta, nv,
+      mp_data[cta], mp_data[cta + 1]);
     int a_count = range.a_count();
     int b_count = range.b_count();
 
-    // Issue the item loads first; they are consumed after the flag setup.
+    // Everything the tile needs from segments[] is fetched first, ahead of
+    // the item loads, so that the start bits can be set while the items are
+    // still in flight and no global load sits on the critical path after
+    // the scan: this thread's start, the start after it, and (thread 0) the
+    // start of the segment that is open when the tile begins.
+    int first_start = 0, first_next = 0, open_start = 0;
+    if(tid < b_count) {
+      int seg = range.b_begin + tid;
+      first_start = segments[seg];
+      first_next = (seg + 1 < num_segments) ? (int)segments[seg + 1] : count;
+    }
+    if(!tid && range.b_begin > 0) open_start = segments[range.b_begin - 1];
+    // The item loads; they are consumed after the flag setup.
     type_t r[chunks][W];
     PRAGMA_UNROLL
     for(int i = 0; i < chunks; ++i) {
@@ -178,10 +278,8 @@ struct segreduce_tile_f {
 
     // One bit per segment start.  Starts of this tile lie in
     // [a_begin, a_end]; the clamp only guards against malformed input.
-    int first_start = 0;
     for(int j = tid; j < b_count; j += nt) {
-      int s = segments[range.b_begin + j];
-      if(j == tid) first_start = s;
+      int s = (j == tid) ? first_start : (int)segments[range.b_begin + j];
       int p = min(max(s - range.a_begin, 0), a_count);
       atomicOr(&shared.flags[p >> 5], 1u << (p & 31));
     }
@@ -216,7 +314,7 @@ struct segreduce_tile_f {
     // Inclusive segmented scan of the thread's items, left to right.
     PRAGMA_UNROLL
     for(int i = 1; i < vt; ++i)
-      x[i] = ((bits >> i) & 1) ? x[i] : op(x[i - 1], x[i]);
+      x[i] = segscan_step_t<op_t, type_t>::step(x[i - 1], x[i], bits, i, op);
 
     PRAGMA_UNROLL
     for(int c = 0; c < chunks; ++c) {
@@ -246,8 +344,11 @@ struct segreduce_tile_f {
     // One thread per segment start of the tile.
     for(int j = tid; j < b_count; j += nt) {
       int seg = range.b_begin + j;
-      int s = (j == tid) ? first_start : segments[seg];
-      int next = (seg + 1 < num_segments) ? segments[seg + 1] : count;
+      int s = first_start, next = first_next;
+      if(j != tid) {
+        s = segments[seg];
+        next = (seg + 1 < num_segments) ? (int)segments[seg + 1] : count;
+      }
       int p = s - range.a_begin;
       if(next <= s) output[seg] = init;                  // empty segment
       else if(p >= 0 && p < a_count) {
@@ -258,28 +359,40 @@ struct segreduce_tile_f {
       // writes it.
     }
 
-    // The segment that was open when the tile began owns items [0, f).
+    // The segment that was open when the tile began owns items [0, f).  Its
+    // code tells the spine which segment to fold the partial into, and
+    // whether that segment already has a value in output[]: it does unless
+    // its start was the very last merged element of its own tile (then that
+    // tile held none of its items and wrote nothing).
     if(!tid) {
       int f = a_count;
       if(b_count) f = min(max(first_start - range.a_begin, 0), a_count);
       if(f > 0 && range.b_begin > 0) {
+        int seg = range.b_begin - 1;
+        int node = open_start + seg;              // merged position of start
+        bool fresh = 0 == (node + 1) % nv;
         carry_values[cta] = fold_to(-1, f - 1);
-        carry_codes[cta] = range.b_begin - 1;
+        carry_codes[cta] = carry_code_t::make(seg, fresh);
       } else {
         carry_values[cta] = init;
-        carry_codes[cta] = -1;
+        carry_codes[cta] = carry_code_t::none;
       }
     }
   }
 };
 
 ////////////////////////////////////////////////////////////////////////////////
-// K3: fold carries into the output.  codes[i] = segment that tile i carried
-// into (-1: none); equal codes are consecutive.  A CTA handles nt carries;
-// the run that is already open at its first carry is passed on to the next
-// level as one carry per CTA.  At the first level tile_begin = the partition
-// array (first item of every tile) decides whether the segment already has a
-// value in output[] (its start tile held some of its items) or not.
+// K3: fold carries into the output, one launch.  codes[i] says which segment
+// tile i carried into (carry_code_t); carries of one segment are consecutive
+// ("a run").  A CTA looks at nt carries.  One segmented scan gives every run
+// that ends among them its fold back to the run's first carry or to the
+// CTA's first carry, whichever comes later.  A run that was already open at
+// the CTA's first carry is completed by the CTA in which it ENDS: its start
+// is known in closed form (the tile after the one that holds the segment's
+// start, at merged position segments[seg] + seg), so that CTA folds the
+// carries in front of its own range cooperatively, in order, straight from
+// global memory.  No CTA ever waits for another and nothing is handed to a
+// second level.
 
 template<int nt, typename output_it, typename segments_it, typename op_t,
   typename type_t>
@@ -289,59 +402,87 @@ struct segreduce_spine_f {
   const int* codes;
   int n;
   segments_it segments;
-  const int* tile_begin;       // null above the first level
+  int nv;
   op_t op;
   type_t init;
-  type_t* values_out;
-  int* codes_out;
 
   MGPU_DEVICE void operator()(int tid, int cta) const {
     typedef cta_segscan_t<nt, type_t> segscan_t;
-    __shared__ typename segscan_t::storage_t shared;
+    typedef cta_reduce_t<nt, type_t> reduce_t;
+    __shared__ union {
+      typename segscan_t::storage_t segscan;
+      typename reduce_t::storage_t reduce;
+    } shared;
+    __shared__ int open_first;
 
-    int gid = nt * cta + tid;
-    int code = (gid < n) ? codes[gid] : -1;
-    int prev = (gid > 0 && gid - 1 < n) ? codes[gid - 1] : -1;
-    int next = (gid + 1 < n) ? codes[gid + 1] : -1;
+    int base = nt * cta;
+    int gid = base + tid;
+    int code = (gid < n) ? codes[gid] : (int)carry_code_t::none;
+    int seg = carry_code_t::seg(code);
+    int prev = (gid > 0 && gid - 1 < n) ?
+      carry_code_t::seg(codes[gid - 1]) : -1;
+    int next = (gid + 1 < n) ? carry_code_t::seg(codes[gid + 1]) : -1;
     type_t value = (gid < n) ? values[gid] : init;
 
-    bool head = code != prev || -1 == code;
-    bool carry_out = -1 != code && code == next;
+    bool head = seg != prev || -1 == seg;
+    bool carry_out = -1 != seg && seg == next;
+    bool run_end = -1 != seg && !carry_out;
+    // Fetch the value to combine with while the scan runs.
+    bool combine = run_end && !carry_code_t::fresh(code);
+    type_t old = init;
+    if(combine) old = output[seg];
+    if(!tid) open_first = -1;
 
     segscan_result_t<type_t> result = segscan_t().segscan(tid, head,
-      carry_out, value, shared, init, op);
+      carry_out, value, shared.segscan, init, op);
+    if(run_end && result.has_carry_in) value = op(result.scan, value);
 
-    bool run_end = -1 != code && (!carry_out || nt - 1 == tid);
-    if(run_end) {
-      if(result.has_carry_in) value = op(result.scan, value);
-      if(result.has_left_head) {
-        // The run started inside this CTA at carry index first.
-        int first = nt * cta + result.left_lane;
-        bool fresh = tile_begin && segments[code] >= tile_begin[first];
-        output[code] = fresh ? value : op(output[code], value);
-      } else {
-        values_out[cta] = value;
-        codes_out[cta] = code;
+    // At most one run is open at `base`; if it ends here, its end thread
+    // publishes where it began.
+    bool open_run = run_end && !result.has_left_head;
+    if(open_run) {
+      int node = segments[seg] + seg;
+      open_first = min(max(node / nv + 1, 0), base);
+    }
+    __syncthreads();
+
+    int first = open_first;
+    if(first >= 0 && first < base) {
+      // Ordered fold of carries [first, base): a contiguous chunk per thread.
+      int len = base - first;
+      int chunk = div_up(len, nt);
+      int active = div_up(len, chunk);
+      int at = first + chunk * tid;
+      type_t x = init;
+      if(tid < active) {
+        // Blocks of eight independent loads, folded in order.
+        x = values[at];
+        for(int k0 = 1; k0 < chunk; k0 += 8) {
+          type_t y[8];
+          PRAGMA_UNROLL
+          for(int k = 0; k < 8; ++k)
+            if(k0 + k < chunk && at + k0 + k < base) y[k] = values[at + k0 + k];
+          PRAGMA_UNROLL
+          for(int k = 0; k < 8; ++k)
+            if(k0 + k < chunk && at + k0 + k < base) x = op(x, y[k]);
+        }
       }
+      type_t front = reduce_t().reduce(tid, x, shared.reduce, active, op, true);
+      if(open_run) value = op(front, value);
     }
-    // No open run at the CTA's first carry: nothing to pass on.
-    if(!tid && (head || -1 == code)) {
-      values_out[cta] = init;
-      codes_out[cta] = -1;
-    }
+
+    if(run_end) output[seg] = combine ? op(old, value) : value;
   }
 };
 
 ////////////////////////////////////////////////////////////////////////////////
 // Workspace layout for one segreduce call (device memory, 256-byte aligned
-// pieces): partitions, tile carries, then the carries of each spine level.
+// pieces): partitions, then one (code, value) carry per tile.
 
 struct segreduce_workspace_t {
-  enum { spine_nt = 1024, max_levels = 4 };
-  int num_ctas, num_partitions, levels;
-  int level_count[max_levels + 1];      // carries entering each level
-  size_t mp_offset, codes_offset[max_levels + 1],
-    values_offset[max_levels + 1], bytes;
+  enum { spine_nt = 256 };
+  int num_ctas, num_partitions;
+  size_t mp_offset, codes_offset, values_offset, bytes;
 
   static size_t align(size_t x) { return (x + 255) & ~(size_t)255; }
 
@@ -352,16 +493,8 @@ struct segreduce_workspace_t {
     num_partitions = num_ctas + 1;
     size_t at = 0;
     mp_offset = at; at = align(at + sizeof(int) * num_partitions);
-    levels = 0;
-    int n = num_ctas;
-    for(;;) {
-      level_count[levels] = n;
-      codes_offset[levels] = at; at = align(at + sizeof(int) * n);
-      values_offset[levels] = at; at = align(at + value_size * n);
-      if(n <= 1 || levels == max_levels) break;
-      n = (n + spine_nt - 1) / spine_nt;
-      ++levels;
-    }
+    codes_offset = at; at = align(at + sizeof(int) * num_ctas);
+    values_offset = at; at = align(at + value_size * num_ctas);
     bytes = at;
   }
 };
@@ -369,7 +502,7 @@ struct segreduce_workspace_t {
 enum {
   phase_partition = 1,    // K1
   phase_tiles = 2,        // K2
-  phase_spine = 4,        // K3, all levels
+  phase_spine = 4,        // K3
   phase_all = 7
 };
 
@@ -389,28 +522,24 @@ void segreduce_launch(input_it input, int count, segments_it segments,
   int* mp_data = (int*)(base + ws.mp_offset);
 
   if(phases & phase_partition)
-    merge_path_partitions_into<bounds_upper>(counting_iterator_t<int>(0),
-      (int64_t)count, segments, (int64_t)num_segments, (int64_t)cta_dim.nv(),
-      less_t<int>(), mp_data, context);
+    load_balance_partitions_into((int64_t)count, segments, num_segments,
+      cta_dim.nv(), mp_data, context);
 
+  type_t* carry_values = (type_t*)(base + ws.values_offset);
+  int* carry_codes = (int*)(base + ws.codes_offset);
   if(phases & phase_tiles) {
     segreduce_tile_f<launch_t, input_it, segments_it, output_it, op_t, type_t>
       k_reduce { input, count, segments, num_segments, output, op, init,
-        mp_data, (type_t*)(base + ws.values_offset[0]),
-        (int*)(base + ws.codes_offset[0]) };
+        mp_data, carry_values, carry_codes };
     cta_launch<launch_t>(k_reduce, ws.num_ctas, context);
   }
 
-  enum { spine_nt = segreduce_workspace_t::spine_nt };
-  for(int level = 0; (phases & phase_spine) && level < ws.levels; ++level) {
-    int n = ws.level_count[level];
+  if((phases & phase_spine) && ws.num_ctas > 1) {
+    enum { spine_nt = segreduce_workspace_t::spine_nt };
     segreduce_spine_f<spine_nt, output_it, segments_it, op_t, type_t>
-      k_spine { output, (const type_t*)(base + ws.values_offset[level]),
-        (const int*)(base + ws.codes_offset[level]), n, segments,
-        level ? (const int*)nullptr : mp_data, op, init,
-        (type_t*)(base + ws.values_offset[level + 1]),
-        (int*)(base + ws.codes_offset[level + 1]) };
-    cta_launch<spine_nt>(k_spine, div_up(n, (int)spine_nt), context);
+      k_spine { output, carry_values, carry_codes, ws.num_ctas, segments,
+        cta_dim.nv(), op, init };
+    cta_launch<spine_nt>(k_spine, div_up(ws.num_ctas, (int)spine_nt), context);
   }
 }
 

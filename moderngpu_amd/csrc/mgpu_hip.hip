@@ -73,9 +73,8 @@ int mgpu_hip_load_balance_partitions(int64_t count, const int* segments,
     count + num_segments >= ((int64_t)1 << 31) || (num_segments && !segments))
     return (int)hipErrorInvalidValue;
   return guarded(stream, [&](context_t& context) {
-    merge_path_partitions_into<bounds_upper>(counting_iterator_t<int>(0),
-      count, segments, (int64_t)num_segments, (int64_t)spacing,
-      less_t<int>(), partitions, context);
+    load_balance_partitions_into(count, segments, num_segments, spacing,
+      partitions, context);
   });
 }
 
