@@ -287,6 +287,23 @@ struct cached_segment_load_t {
     value_t data[nt];
   };
 
+  // Stages the values of segments [begin, begin + count) in LDS if they fit
+  // (one coalesced global read per segment); ends with a barrier then.
+  // `count` must be the same in every thread.
+  MGPU_DEVICE static bool stage(int tid, int begin, int count,
+    storage_t& storage, pointers_t iterators) {
+    if(count > nt) return false;
+    if(tid < count && begin + tid >= 0)
+      storage.data[tid] = mgpu::load(iterators, begin + tid);
+    __syncthreads();
+    return true;
+  }
+  // Value of segment seg = begin + rel.
+  MGPU_DEVICE static value_t get(bool staged, int rel, int seg,
+    const storage_t& storage, pointers_t iterators) {
+    return staged ? storage.data[rel] : mgpu::load(iterators, max(seg, 0));
+  }
+
   // range = segments the tile's items can belong to.
   template<int vt0, int vt>
   MGPU_DEVICE static array_t<value_t, vt> load(int tid, int count,
@@ -315,6 +332,13 @@ template<int nt>
 struct cached_segment_load_t<nt, tuple<> > {
   typedef empty_t storage_t;
   typedef tuple<> value_t;
+
+  MGPU_DEVICE static bool stage(int, int, int, storage_t&, tuple<>) {
+    return false;
+  }
+  MGPU_DEVICE static value_t get(bool, int, int, const storage_t&, tuple<>) {
+    return value_t();
+  }
 
   template<int vt0, int vt>
   MGPU_DEVICE static array_t<value_t, vt> load(int, int, range_t,

@@ -6,6 +6,37 @@
 
 BEGIN_MGPU_NAMESPACE
 
+namespace detail {
+// output[index] = value of the item's segment, for any output iterator ...
+template<typename type_t, typename output_it>
+struct interval_expand_f {
+  output_it output;
+  MGPU_DEVICE void operator()(int index, int, int,
+    tuple<type_t> desc) const {
+    output[index] = get<0>(desc);
+  }
+};
+// ... and, for pointers, W values per call written with the widest stores
+// the element type allows.
+template<typename type_t>
+struct interval_expand_f<type_t, type_t*> {
+  typedef void chunk_functor_tag;
+  type_t* output;
+  MGPU_DEVICE void operator()(int index, int, int,
+    tuple<type_t> desc) const {
+    output[index] = get<0>(desc);
+  }
+  template<int W>
+  MGPU_DEVICE void chunk(int index, const int (&)[W], const int (&)[W],
+    const tuple<type_t> (&desc)[W]) const {
+    type_t x[W];
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) x[e] = get<0>(desc[e]);
+    store_consecutive<W>(output + index, x);
+  }
+};
+} // namespace detail
+
 // output[index] = input[segment of index]: each per-segment value is
 // replicated over the segment's items.
 template<typename launch_arg_t = empty_t, typename input_it,
@@ -15,12 +46,8 @@ void interval_expand(input_it input, int count, segments_it segments,
 
   typedef typename std::iterator_traits<input_it>::value_type type_t;
   transform_lbs<launch_arg_t>(
-    []MGPU_DEVICE(int index, int, int, tuple<type_t> desc,
-      output_it output) {
-      output[index] = get<0>(desc);
-    },
-    count, segments, num_segments, make_tuple(input), context, output
-  );
+    detail::interval_expand_f<type_t, output_it> { output },
+    count, segments, num_segments, make_tuple(input), context);
 }
 
 // output[index] = input[gather[seg] + rank].

@@ -21,6 +21,39 @@ namespace detail {
 // SIMD) x 16 items.
 typedef launch_box_t<arch_gfx950_cta<256, 16, 16> > lbs_launch_default_t;
 
+// A functor may take W consecutive work-items per call instead of one:
+//   typedef void chunk_functor_tag;
+//   template<int W, typename value_t, typename... args_t>
+//   void chunk(int index, const int (&seg)[W], const int (&rank)[W],
+//     const value_t (&cached)[W], args_t...) const;
+// next to the per-item operator() (still used at the ragged end of a tile).
+// The library's own load_balance_search / interval_expand functors do, so
+// that each lane issues 16-byte stores.
+template<typename func_t, typename enable_t = void>
+struct is_chunk_functor_t : std::false_type { };
+template<typename func_t>
+struct is_chunk_functor_t<func_t,
+  typename std::conditional<false, typename func_t::chunk_functor_tag,
+    void>::type> : std::true_type { };
+
+// Stores W consecutive elements.  Element types whose size is a multiple of
+// four bytes go out as 16-byte stores (global_store_dwordx4 only needs dword
+// alignment); smaller ones element by element.
+template<int W, typename type_t>
+MGPU_DEVICE inline void store_consecutive(type_t* dest,
+  const type_t (&x)[W]) {
+  if constexpr(0 == sizeof(type_t) % 4 && W * sizeof(type_t) <= 64) {
+    enum { words = W * sizeof(type_t) / 4 };
+    typedef unsigned v_t __attribute__((ext_vector_type(words), aligned(4)));
+    v_t v;
+    __builtin_memcpy(&v, x, sizeof(v));
+    *(v_t*)dest = v;
+  } else {
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) dest[e] = x[e];
+  }
+}
+
 template<typename launch_t, typename func_t, typename segments_it,
   typename pointers_t, typename int_t>
 struct transform_lbs_f {
@@ -34,29 +67,87 @@ struct transform_lbs_f {
   template<typename... args_t>
   MGPU_DEVICE void operator()(int tid, int cta, args_t... args) const {
     typedef typename launch_t::sm_ptx params_t;
-    enum { nt = params_t::nt, vt = params_t::vt, vt0 = params_t::vt0 };
+    enum { nt = params_t::nt, vt = params_t::vt };
     typedef cta_load_balance_t<nt, vt> load_balance_t;
+    typedef typename load_balance_t::layout_t layout_t;
     typedef cached_segment_load_t<nt, pointers_t> cached_load_t;
     typedef typename cached_load_t::value_t value_t;
+    enum { W = load_balance_t::W, chunks = vt / W };
 
     __shared__ struct {
       typename load_balance_t::storage_t lbs;
       typename cached_load_t::storage_t cached;
     } shared;
 
-    auto lbs = load_balance_t().load_balance(count, segments, num_segments,
-      tid, cta, mp_data, shared.lbs);
+    // After fill(), LDS slot p holds (segment of tile item p) - seg_base and
+    // the tile's segment starts sit behind the slots.
+    merge_range_t range = load_balance_t().fill(count, segments,
+      num_segments, tid, cta, mp_data, shared.lbs);
+    int a_count = range.a_count();
+    int seg_base = range.b_begin - 1;
+    const int* slots = shared.lbs.indices;
+    const int* starts = slots + load_balance_t::starts_offset(a_count);
 
-    // Items of the tile belong to segments [b_begin - 1, b_end).
-    range_t seg_range { lbs.merge_range.b_begin - 1, lbs.merge_range.b_end };
-    array_t<value_t, vt> cached_values = cached_load_t::template load<vt0>(
-      tid, lbs.merge_range.a_count(), seg_range, lbs.segments,
+    // Items of the tile belong to segments [seg_base, b_end): fetch their
+    // cached values once into LDS when they fit.
+    bool staged = cached_load_t::stage(tid, seg_base, range.b_count() + 1,
       shared.cached, caching_iterators);
 
-    strided_iterate<nt, vt, vt0>([&](int i, int) {
-      f(lbs.indices[i], lbs.segments[i], lbs.ranks[i], cached_values[i],
-        args...);
-    }, tid, lbs.merge_range.a_count());
+    // The emission loop exists twice -- cached values staged in LDS, or
+    // gathered from global memory -- so that each copy is straight-line code.
+    auto emit_all = [&](auto staged_tag) {
+      if constexpr(is_chunk_functor_t<func_t>::value) {
+        // The functor consumes W consecutive items at a time (one 16-byte
+        // store per chunk for 4-byte results).  Chunk nt * i + tid in step i:
+        // consecutive lanes own consecutive chunks.
+        PRAGMA_UNROLL
+        for(int i = 0; i < chunks; ++i) {
+          int p = W * (nt * i + tid);
+          int index = range.a_begin + p;
+          if(p + W <= a_count) {
+            int rel[W], seg[W], rank[W];
+            value_t cached[W];
+            lds_load_chunk<W>(slots + layout_t::index(p), rel);
+            PRAGMA_UNROLL
+            for(int e = 0; e < W; ++e) {
+              seg[e] = seg_base + rel[e];
+              rank[e] = index + e - starts[rel[e]];
+              cached[e] = cached_load_t::get(decltype(staged_tag)::value, rel[e], seg[e],
+                shared.cached, caching_iterators);
+            }
+            f.template chunk<W>(index, seg, rank, cached, args...);
+          } else {
+            PRAGMA_UNROLL
+            for(int e = 0; e < W; ++e) {
+              if(p + e < a_count) {
+                int rel = slots[layout_t::index(p + e)];
+                int seg = seg_base + rel;
+                f(index + e, seg, index + e - starts[rel],
+                  cached_load_t::get(decltype(staged_tag)::value, rel, seg, shared.cached,
+                    caching_iterators), args...);
+              }
+            }
+          }
+        }
+      } else {
+        // One item per call, item nt * i + tid in step i: whatever the functor
+        // stores per item is coalesced across the wavefront.
+        PRAGMA_UNROLL
+        for(int i = 0; i < vt; ++i) {
+          int p = nt * i + tid;
+          if(p < a_count) {
+            int rel = slots[layout_t::index(p)];
+            int seg = seg_base + rel;
+            int index = range.a_begin + p;
+            f(index, seg, index - starts[rel],
+              cached_load_t::get(decltype(staged_tag)::value, rel, seg, shared.cached,
+                caching_iterators), args...);
+          }
+        }
+      }
+    };
+    if(staged) emit_all(std::true_type());
+    else emit_all(std::false_type());
   }
 };
 
@@ -119,11 +210,26 @@ void transform_lbs(func_t f, int count, segments_it segments,
 }
 
 namespace detail {
+// output[index] = seg, for any output iterator ...
 template<typename output_it>
 struct lbs_store_seg_f {
   output_it output;
-  MGPU_DEVICE void operator()(int index, int seg, int) const {
+  MGPU_DEVICE void operator()(int index, int seg, int, tuple<>) const {
     output[index] = seg;
+  }
+};
+// ... and, for int pointers, W segments per 16-byte store.
+template<>
+struct lbs_store_seg_f<int*> {
+  typedef void chunk_functor_tag;
+  int* output;
+  MGPU_DEVICE void operator()(int index, int seg, int, tuple<>) const {
+    output[index] = seg;
+  }
+  template<int W>
+  MGPU_DEVICE void chunk(int index, const int (&seg)[W], const int (&)[W],
+    const tuple<> (&)[W]) const {
+    store_consecutive<W>(output + index, seg);
   }
 };
 } // namespace detail
@@ -134,7 +240,7 @@ template<typename launch_arg_t = empty_t, typename segments_it,
 void load_balance_search(int count, segments_it segments,
   int num_segments, output_it output, context_t& context) {
   transform_lbs<launch_arg_t>(detail::lbs_store_seg_f<output_it> { output },
-    count, segments, num_segments, context);
+    count, segments, num_segments, tuple<>(), context);
 }
 
 END_MGPU_NAMESPACE

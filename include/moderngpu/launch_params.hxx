@@ -16,10 +16,15 @@
 
 #define MGPU_LAUNCH_PARAMS(launch_box) \
   typename launch_box::MGPU_SM_TAG
-// HIP's second __launch_bounds__ argument is "min waves per EU", not CUDA's
-// "min blocks per SM", so the occupancy hint of CUDA boxes is not forwarded.
+// The fourth launch parameter (occ) is the minimum number of wavefronts per
+// SIMD the kernel should stay resident with (0: no constraint); the register
+// allocator is told to stay within that budget.  CUDA boxes written with
+// "min blocks per SM" in that slot reach gfx950 only through inheritance;
+// arch_gfx950_cta<nt, vt, vt0, occ> states it in CDNA terms.
 #define MGPU_LAUNCH_BOUNDS(launch_box) \
-  __launch_bounds__(launch_box::sm_ptx::nt)
+  __launch_bounds__(launch_box::sm_ptx::nt) \
+  __attribute__((amdgpu_waves_per_eu(launch_box::sm_ptx::occ > 8 ? 0 : \
+    launch_box::sm_ptx::occ)))
 
 BEGIN_MGPU_NAMESPACE
 

@@ -38,21 +38,10 @@ struct store_seg_rank_f {
   }
 };
 
-struct store_seg_f {
-  int* output;
-  MGPU_DEVICE void operator()(int index, int seg, int, tuple<>) const {
-    output[index] = seg;
-  }
-};
+typedef detail::lbs_store_seg_f<int*> store_seg_f;
 
 template<typename type_t>
-struct expand_f {
-  type_t* output;
-  MGPU_DEVICE void operator()(int index, int, int,
-    tuple<type_t> desc) const {
-    output[index] = get<0>(desc);
-  }
-};
+using expand_f = detail::interval_expand_f<type_t, type_t*>;
 template<typename type_t>
 struct gather_f {
   const type_t* input; type_t* output;
