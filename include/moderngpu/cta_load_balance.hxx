@@ -72,6 +72,27 @@ struct chunk_width_t {
   };
 };
 
+// Which tile a CTA works on.  The hardware hands consecutive workgroups of a
+// grid to the 8 accelerator dies (XCDs) of the package in turn, and each XCD
+// has its own L2.  With tile == blockIdx.x, neighbouring tiles -- which share
+// the cache line where one tile's data ends and the next begins -- always sit
+// on different XCDs: the line is fetched twice, or written back partially by
+// two L2s.  Here each XCD takes runs of xcd_run consecutive tiles, and the
+// runs of the 8 XCDs interleave, so the set of tiles in flight stays one
+// compact window of memory.  (Giving each XCD one contiguous eighth of all
+// tiles merges even more boundary lines and is the fastest layout for a pure
+// store kernel, but measured slower for these kernels, which read and write
+// at the same time.)  The grid must be xcd_grid(num_tiles); CTAs whose tile
+// is >= num_tiles have nothing to do.
+enum { num_xcds = 8, xcd_run = 16 };
+MGPU_HOST_DEVICE int xcd_grid(int num_tiles) {
+  return div_up(num_tiles, (int)(num_xcds * xcd_run)) * (num_xcds * xcd_run);
+}
+MGPU_DEVICE inline int xcd_tile(int cta, int) {
+  int xcd = cta % num_xcds, local = cta / num_xcds;
+  return ((local / xcd_run) * num_xcds + xcd) * xcd_run + local % xcd_run;
+}
+
 // The tile's item and segment ranges from the two splits at its ends, forced
 // to be consistent: each split inside what its cross-diagonal allows, ends not
 // before begins, at most nv elements.  For well-formed input (ascending

@@ -63,9 +63,12 @@ struct transform_lbs_f {
   int num_segments;
   pointers_t caching_iterators;
   const int_t* mp_data;
+  int num_tiles;
 
   template<typename... args_t>
   MGPU_DEVICE void operator()(int tid, int cta, args_t... args) const {
+    int tile = xcd_tile(cta, num_tiles);
+    if(tile >= num_tiles) return;
     typedef typename launch_t::sm_ptx params_t;
     enum { nt = params_t::nt, vt = params_t::vt };
     typedef cta_load_balance_t<nt, vt> load_balance_t;
@@ -82,7 +85,7 @@ struct transform_lbs_f {
     // After fill(), LDS slot p holds (segment of tile item p) - seg_base and
     // the tile's segment starts sit behind the slots.
     merge_range_t range = load_balance_t().fill(count, segments,
-      num_segments, tid, cta, mp_data, shared.lbs);
+      num_segments, tid, tile, mp_data, shared.lbs);
     int a_count = range.a_count();
     int seg_base = range.b_begin - 1;
     const int* slots = shared.lbs.indices;
@@ -171,9 +174,11 @@ void transform_lbs_launch(func_t f, int count, segments_it segments,
       launch_t::nv(context), mp_data, context);
 
   if(phases & lbs_phase_tiles) {
+    int num_tiles = launch_t::cta_dim(context).num_ctas(count + num_segments);
     transform_lbs_f<launch_t, func_t, segments_it, pointers_t, int>
-      k { f, count, segments, num_segments, caching_iterators, mp_data };
-    cta_transform<launch_t>(k, count + num_segments, context, args...);
+      k { f, count, segments, num_segments, caching_iterators, mp_data,
+        num_tiles };
+    cta_launch<launch_t>(k, xcd_grid(num_tiles), context, args...);
   }
 }
 

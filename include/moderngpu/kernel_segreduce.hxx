@@ -179,13 +179,17 @@ struct segscan_step_t<minimum_t<type_t>, type_t,
   segscan_select_step_t<minimum_t<type_t>, type_t> { };
 
 ////////////////////////////////////////////////////////////////////////////////
-// Default tiles on gfx950, by value size.
+// Default tiles on gfx950: 256 threads x 16 values for 4- and 8-byte values
+// (16 KB / 32 KB of values in LDS); wider value types get fewer values per
+// thread so that the tile stays under the 64 KB a workgroup may declare.
 
 template<typename type_t>
 struct segreduce_launch_default_t {
-  typedef launch_box_t<
-    arch_gfx950_cta<256, (sizeof(type_t) > 4 ? 8 : 16)>
-  > type_t_;
+  enum {
+    vt = sizeof(type_t) <= 8 ? 16 :
+      (128 / sizeof(type_t) > 1 ? 128 / sizeof(type_t) : 1)
+  };
+  typedef launch_box_t<arch_gfx950_cta<256, vt> > type_t_;
 };
 
 ////////////////////////////////////////////////////////////////////////////////
@@ -221,8 +225,12 @@ struct segreduce_tile_f {
   const int* mp_data;
   type_t* carry_values;
   int* carry_codes;
+  int num_tiles;
 
   MGPU_DEVICE void operator()(int tid, int cta) const {
+    // Neighbouring tiles run on the same XCD (see xcd_tile).
+    cta = xcd_tile(cta, num_tiles);
+    if(cta >= num_tiles) return;
     typedef typename launch_t::sm_ptx params_t;
     enum {
       nt = params_t::nt, vt = params_t::vt, nv = nt * vt,
@@ -530,8 +538,8 @@ void segreduce_launch(input_it input, int count, segments_it segments,
   if(phases & phase_tiles) {
     segreduce_tile_f<launch_t, input_it, segments_it, output_it, op_t, type_t>
       k_reduce { input, count, segments, num_segments, output, op, init,
-        mp_data, carry_values, carry_codes };
-    cta_launch<launch_t>(k_reduce, ws.num_ctas, context);
+        mp_data, carry_values, carry_codes, ws.num_ctas };
+    cta_launch<launch_t>(k_reduce, xcd_grid(ws.num_ctas), context);
   }
 
   if((phases & phase_spine) && ws.num_ctas > 1) {
