@@ -252,7 +252,13 @@ FACTORIES = {
 # HBM traffic of the dominant kernel per launch, from rocprofv3 --pmc
 # FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by what the same counters
 # read for a plain copy of known size.  None until measured.
-TRAFFIC_BYTES = {}
+TRAFFIC_BYTES = {
+    # profiles/segreduce_tile_f__c2_segreduce_f32.md: FETCH 133,562.5 KiB x 2.000
+    # + WRITE 4,279.3 KiB x 1.000
+    "c2_segreduce_f32": int((133562.5 * 2.000 + 4279.3) * 1024),
+    # profiles/transform_lbs_f__c3_load_balance_search.md
+    "c3_load_balance_search": int((33634.5 * 2.000 + 1048977.7) * 1024),
+}
 
 
 def time_steps(fn, steps, warmup):
@@ -311,6 +317,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--extra", default="c3_load_balance_search",
                     help="comma-separated further workloads reported under 'others'")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="only run a plain 256 MiB device copy a few times: the kernel of "
+                         "known traffic that rocprofv3 FETCH_SIZE/WRITE_SIZE are scaled by")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: every box of this build has one, and the "
@@ -320,6 +329,19 @@ def main():
     if not torch.cuda.is_available():
         sys.exit("bench.py needs a GPU")
     torch.cuda.set_device(0)
+
+    if args.copy_calibration:
+        n = (256 << 20) // 4
+        src = torch.rand(n, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        junk = torch.empty(3 * n, dtype=torch.float32, device="cuda")
+        for _ in range(args.steps):
+            junk.zero_()                 # push src/dst out of the 256 MB memory-side cache
+            dst.copy_(src)
+        torch.cuda.synchronize()
+        print(json.dumps({"calibration": "torch copy_", "bytes_read": n * 4,
+                          "bytes_written": n * 4, "launches": args.steps}))
+        return
 
     def measure(key, with_cpu):
         wk = FACTORIES[key](args.copies)
