@@ -96,7 +96,7 @@ def make_c3(copies, expand=False):
         wk.key = "c3_interval_expand_i32"
         wk.name = "interval_expand int32, 2^24 Zipf(1.2) segments, 2^28 items"
         wk.bytes = s * 4 + s * 4 + n * 4
-        wk.kernel = "transform_lbs_f<256x16, expand>"
+        wk.kernel = "transform_lbs_f<512x12, expand>"
         wk.step = lambda i: m.interval_expand(vals[i % copies], n, segs[i % copies],
                                               out=outs[i % copies])
         wk.tiles = lambda i: m.interval_expand(vals[i % copies], n, segs[i % copies],
@@ -105,7 +105,7 @@ def make_c3(copies, expand=False):
         wk.key = "c3_load_balance_search"
         wk.name = "load_balance_search, 2^24 Zipf(1.2) segments, 2^28 items"
         wk.bytes = s * 4 + n * 4
-        wk.kernel = "transform_lbs_f<256x16, store seg>"
+        wk.kernel = "transform_lbs_f<512x12, store seg>"
         wk.step = lambda i: m.load_balance_search(n, segs[i % copies], out=outs[i % copies])
         wk.tiles = lambda i: m.load_balance_search(n, segs[i % copies], out=outs[i % copies],
                                                    phases=2)

@@ -53,8 +53,9 @@ enum { MGPU_PHASE_PARTITION = 1, MGPU_PHASE_TILES = 2, MGPU_PHASE_SPINE = 4,
 MGPU_HIP_API int mgpu_hip_version(void);
 /* Text for a return code (hipGetErrorString). */
 MGPU_HIP_API const char* mgpu_hip_error_string(int code);
-/* Tile size nv = nt * vt (merged elements per CTA) the library uses for
- * segreduce on `dtype`, and for the load-balancing search. */
+/* Merged elements (items + segment starts) between consecutive tile splits:
+ * what the library uses as `spacing` for segreduce on `dtype`, and for the
+ * load-balancing search. */
 MGPU_HIP_API int mgpu_hip_segreduce_tile_size(int dtype);
 MGPU_HIP_API int mgpu_hip_lbs_tile_size(void);
 

@@ -112,6 +112,39 @@ MGPU_DEVICE inline merge_range_t tile_range(int count, int num_segments,
   return r;
 }
 
+// Tile ends moved onto 128-byte lines of a 4-byte output.
+//
+// With splits taken exactly on the cross-diagonals, a tile's items begin and
+// end anywhere, so the first and last cache line of what a CTA stores per item
+// are shared with its neighbours and every 16-byte store straddles two
+// 16-byte slots.  A split (a, b) may however be moved back along the merge
+// path to any earlier point of the path without changing any result; the
+// partition kernel of the search (load_balance_partitions_snapped) moves it
+// to the last point whose item index is a multiple of lbs_snap_items, unless
+// lbs_snap_window or more segment starts would have to move with it.  A moved
+// split retreats by at most (lbs_snap_items - 1) + (lbs_snap_window - 1)
+// merged elements, so tiles cut at multiples of lbs_tile_spacing(nv) =
+// nv - lbs_snap_slack never exceed nv elements.
+enum { lbs_snap_items = 32, lbs_snap_window = 32, lbs_snap_slack = 64 };
+
+MGPU_HOST_DEVICE constexpr int lbs_tile_spacing(int nv) {
+  return nv >= 8 * lbs_snap_slack ? nv - lbs_snap_slack : nv;
+}
+
+// Range of a tile from the snapped splits at its two ends, pairs[2 * i] =
+// items and pairs[2 * i + 1] = starts in front of split i, made consistent
+// the way tile_range() does (this only matters for malformed input).
+MGPU_DEVICE inline merge_range_t paired_tile_range(int count,
+  int num_segments, int tile, int nv, const int* pairs) {
+  int a0 = pairs[2 * tile], b0 = pairs[2 * tile + 1];
+  int a1 = pairs[2 * tile + 2], b1 = pairs[2 * tile + 3];
+  a0 = min(max(a0, 0), count);
+  b0 = min(max(b0, 0), num_segments);
+  a1 = min(min(max(a1, a0), a0 + nv), count);
+  b1 = min(min(max(b1, b0), b0 + nv - (a1 - a0)), num_segments);
+  return merge_range_t { a0, a1, b0, b1 };
+}
+
 // Read W consecutive LDS elements starting at an index that is a multiple
 // of W.
 template<int W, typename type_t>
@@ -191,6 +224,15 @@ struct cta_load_balance_t {
 
     merge_range_t range = detail::tile_range(count, num_segments, cta, nv,
       partitions[cta], partitions[cta + 1]);
+    fill(range, segments, tid, storage);
+    return range;
+  }
+
+  // Same for a tile whose range the caller has worked out.
+  template<typename segments_it>
+  MGPU_DEVICE void fill(merge_range_t range, segments_it segments, int tid,
+    storage_t& storage) const {
+
     int a_count = range.a_count();
     int b_count = range.b_count();
     int* slots = storage.indices;
@@ -253,7 +295,6 @@ struct cta_load_balance_t {
           slots + layout_t::index(vt * tid + W * c), chunk);
     }
     __syncthreads();
-    return range;
   }
 
   // Full search: (index, segment, rank) per item in strided order.  Items

@@ -17,9 +17,9 @@ BEGIN_MGPU_NAMESPACE
 
 namespace detail {
 
-// Default tile for the search on gfx950: 256 threads (one wavefront per
-// SIMD) x 16 items.
-typedef launch_box_t<arch_gfx950_cta<256, 16, 16> > lbs_launch_default_t;
+// Default tile for the search on gfx950: 512 threads (two wavefronts per
+// SIMD) x 12 items, 24 KB of item slots per CTA.
+typedef launch_box_t<arch_gfx950_cta<512, 12, 12> > lbs_launch_default_t;
 
 // A functor may take W consecutive work-items per call instead of one:
 //   typedef void chunk_functor_tag;
@@ -84,8 +84,9 @@ struct transform_lbs_f {
 
     // After fill(), LDS slot p holds (segment of tile item p) - seg_base and
     // the tile's segment starts sit behind the slots.
-    merge_range_t range = load_balance_t().fill(count, segments,
-      num_segments, tid, tile, mp_data, shared.lbs);
+    merge_range_t range = paired_tile_range(count, num_segments, tile,
+      load_balance_t::nv, mp_data);
+    load_balance_t().fill(range, segments, tid, shared.lbs);
     int a_count = range.a_count();
     int seg_base = range.b_begin - 1;
     const int* slots = shared.lbs.indices;
@@ -160,8 +161,14 @@ namespace detail {
 
 enum { lbs_phase_partition = 1, lbs_phase_tiles = 2, lbs_phase_all = 3 };
 
+// Ints of partition storage for `total` merged elements cut into tiles of nv:
+// one (items, starts) pair per split.
+MGPU_HOST_DEVICE inline size_t lbs_partition_ints(int total, int nv) {
+  return 2 * ((size_t)div_up(total, lbs_tile_spacing(nv)) + 1);
+}
+
 // Partition + tile kernels with the partition array in caller-provided
-// device memory (div_up(count + num_segments, nv) + 1 ints).
+// device memory: lbs_partition_ints(count + num_segments, nv) ints.
 template<typename launch_t, typename func_t, typename segments_it,
   typename pointers_t, typename... args_t>
 void transform_lbs_launch(func_t f, int count, segments_it segments,
@@ -169,12 +176,13 @@ void transform_lbs_launch(func_t f, int count, segments_it segments,
   context_t& context, args_t... args) {
 
   if(count + num_segments <= 0) return;
+  int spacing = lbs_tile_spacing(launch_t::nv(context));
   if(phases & lbs_phase_partition)
-    load_balance_partitions_into((int64_t)count, segments, num_segments,
-      launch_t::nv(context), mp_data, context);
+    load_balance_partitions_snapped<lbs_snap_items, lbs_snap_window>(count,
+      segments, num_segments, spacing, mp_data, context);
 
   if(phases & lbs_phase_tiles) {
-    int num_tiles = launch_t::cta_dim(context).num_ctas(count + num_segments);
+    int num_tiles = div_up(count + num_segments, spacing);
     transform_lbs_f<launch_t, func_t, segments_it, pointers_t, int>
       k { f, count, segments, num_segments, caching_iterators, mp_data,
         num_tiles };
@@ -194,8 +202,8 @@ void transform_lbs(func_t f, int count, segments_it segments,
     detail::lbs_launch_default_t>::type_t launch_t;
 
   if(count + num_segments <= 0) return;
-  int num_partitions = div_up(count + num_segments, launch_t::nv(context)) + 1;
-  mem_t<int> mp(num_partitions, context);
+  mem_t<int> mp(detail::lbs_partition_ints(count + num_segments,
+    launch_t::nv(context)), context);
   detail::transform_lbs_launch<launch_t>(f, count, segments, num_segments,
     caching_iterators, mp.data(), detail::lbs_phase_all, context, args...);
 }

@@ -71,6 +71,28 @@ struct merge_path_partition_f {
   }
 };
 
+// Division of a non-negative int by a fixed positive divisor without the
+// integer-division sequence: a shift for powers of two, else one 32x32->64
+// multiply by magic = floor(2^(31 + s) / d) + 1 with s = ceil(log2 d), which
+// gives the exact quotient for every dividend below 2^31.
+struct int_divider_t {
+  unsigned magic;       // 0: divisor is a power of two
+  int shift;
+
+  static int_divider_t make(int d) {
+    int s = 0;
+    while(((int64_t)1 << s) < d) ++s;
+    if(((int64_t)1 << s) == d) return int_divider_t { 0u, s };
+    uint64_t m = (((uint64_t)1 << (31 + s)) / (uint64_t)d) + 1;
+    return int_divider_t { (unsigned)m, s - 1 };
+  }
+  MGPU_HOST_DEVICE int div(int n) const {
+    return magic ?
+      (int)((unsigned)(((uint64_t)(unsigned)n * magic) >> 32) >> shift) :
+      (n >> shift);
+  }
+};
+
 // Kernel body of load_balance_partitions.  The merge of item indices with
 // segment starts has a closed form: the start of segment j sits at merged
 // position m_j = segments[j] + j (all items before it plus all starts before
@@ -81,18 +103,46 @@ struct merge_path_partition_f {
 // boundaries that fall between a start and the next one: none for most
 // segments, one for a segment that straddles a boundary, many for a segment
 // that spans tiles (long runs are queued in LDS and written by the whole CTA).
-template<int nt, typename int_t, typename segments_it>
+//
+// With snap > 0 the kernel writes pairs (a, b) = (items, starts) in front of
+// each split instead of a alone, and moves every split except the first and
+// the last back along the merge path to the nearest earlier point whose item
+// index is a multiple of snap -- the tile kernels of the load-balancing
+// search then store whole cache lines.  Moving from a to a' = a - a % snap
+// also hands back the starts in (a', a]; if there are `window` or more of
+// them the split stays where it is.  A moved split retreats by at most
+// (snap - 1) + (window - 1) merged elements.
+template<int nt, typename int_t, typename segments_it, int snap = 0,
+  int window = 32>
 struct lbs_partition_scatter_f {
   enum { vt = 4, direct = 8 };
   segments_it segments;
   int num_segments;
   int count;
   int spacing;
-  int shift;            // log2(spacing) if it is a power of two, else -1
+  int_divider_t by_spacing;
   int_t* p;
 
   MGPU_DEVICE int tile_of(int merged) const {
-    return shift >= 0 ? (merged >> shift) : merged / spacing;
+    return by_spacing.div(merged);
+  }
+
+  // Split `boundary` with `before` starts in front of it, where the last of
+  // those starts (segment before - 1) is known not to lie behind the snapped
+  // item index.
+  MGPU_DEVICE void write_inside(int boundary, int before) const {
+    int a = boundary * spacing - before;
+    if constexpr(snap > 0) {
+      if(boundary * spacing < count + num_segments) a -= a % snap;
+      p[2 * boundary] = (int_t)a;
+      p[2 * boundary + 1] = (int_t)before;
+    } else
+      p[boundary] = (int_t)a;
+  }
+
+  MGPU_DEVICE void write_pair(int boundary, int a, int before) const {
+    p[2 * boundary] = (int_t)a;
+    p[2 * boundary + 1] = (int_t)before;
   }
 
   MGPU_DEVICE void operator()(int tid, int cta) const {
@@ -125,24 +175,62 @@ struct lbs_partition_scatter_f {
 
     // Boundaries b with m_j < spacing * b <= m_{j+1} have exactly j + 1
     // starts in front of them.  The clamps keep malformed (unsorted) input
-    // from writing outside p.
+    // from writing outside p.  Only the first of them can be closer than
+    // `snap` items to the start of segment j; all threads of a wavefront
+    // stay together here so that they can resolve those cases jointly.
+    int lane = tid % warp_size;
+    // tile_at[e] = tile holding merged position m_{j0 + e}.
+    int tile_at[vt + 1];
+    PRAGMA_UNROLL
+    for(int e = 0; e <= vt; ++e)
+      tile_at[e] = tile_of(min(max(starts[e] + j0 + e, 0), total));
+
     PRAGMA_UNROLL
     for(int e = 0; e < vt; ++e) {
       int j = j0 + e;
-      if(j >= num_segments) break;
-      int m0 = min(max(starts[e] + j, 0), total);
-      int m1 = min(max(starts[e + 1] + j + 1, 0), total);
-      int first = tile_of(m0) + 1;
-      int n = tile_of(m1) - first + 1;
-      if(n <= 0) continue;
-      if(n <= direct) {
-        for(int k = 0; k < n; ++k)
-          p[first + k] = (int_t)((first + k) * spacing - (j + 1));
-      } else {
-        int slot = atomicAdd(&queue_size, 1);
-        queue[slot][0] = first;
-        queue[slot][1] = n;
-        queue[slot][2] = j + 1;
+      int first = 0, n = 0;
+      if(j < num_segments) {
+        first = tile_at[e] + 1;
+        n = max(tile_at[e + 1] - first + 1, 0);
+      }
+
+      if constexpr(snap > 0) {
+        // First split: the snapped item index may lie in front of the start
+        // of segment j and of starts before it.  The wavefront counts them
+        // for one such split at a time: lane l looks at start j - l.
+        int a = first * spacing - (j + 1);
+        int a_snap = a - a % snap;
+        bool inner = n > 0 && first * spacing < total;
+        bool look = inner && starts[e] > a_snap;
+        int back = 0;
+        lanemask_t pending = ballot(look);
+        while(pending) {
+          int src = (int)__builtin_ctzll(pending);
+          pending &= pending - 1;
+          int src_j = readlane(j, src);
+          int src_snap = readlane(a_snap, src);
+          int idx = src_j - lane;
+          bool later = lane < window && idx >= 0 &&
+            (int)segments[idx] > src_snap;
+          int c = __builtin_popcountll(ballot(later));
+          if(lane == src) back = c;
+        }
+        if(n > 0) {
+          if(inner && back < window) write_pair(first, a_snap, j + 1 - back);
+          else write_pair(first, a, j + 1);
+        }
+      } else if(n > 0)
+        write_inside(first, j + 1);
+
+      if(n > 1) {
+        if(n <= direct) {
+          for(int k = 1; k < n; ++k) write_inside(first + k, j + 1);
+        } else {
+          int slot = atomicAdd(&queue_size, 1);
+          queue[slot][0] = first + 1;
+          queue[slot][1] = n - 1;
+          queue[slot][2] = j + 1;
+        }
       }
     }
     __syncthreads();
@@ -150,13 +238,18 @@ struct lbs_partition_scatter_f {
     int queued = queue_size;
     for(int q = 0; q < queued; ++q) {
       int first = queue[q][0], n = queue[q][1], before = queue[q][2];
-      for(int k = tid; k < n; k += nt)
-        p[first + k] = (int_t)((first + k) * spacing - before);
+      for(int k = tid; k < n; k += nt) write_inside(first + k, before);
     }
 
     if(!cta && !tid) {
-      p[0] = 0;
-      p[div_up(total, spacing)] = (int_t)count;
+      int last = div_up(total, spacing);
+      if constexpr(snap > 0) {
+        p[0] = 0; p[1] = 0;
+        p[2 * last] = (int_t)count; p[2 * last + 1] = (int_t)num_segments;
+      } else {
+        p[0] = 0;
+        p[last] = (int_t)count;
+      }
     }
   }
 };
@@ -192,9 +285,40 @@ int load_balance_partitions_into(int64_t count, segments_it segments,
     return merge_path_partitions_into<bounds_upper>(
       counting_iterator_t<int_t>(0), count, segments, (int64_t)0,
       (int64_t)spacing, less_t<int_t>(), p, context);
-  int shift = is_pow2(spacing) ? s_log2(spacing) : -1;
   detail::lbs_partition_scatter_f<nt, int_t, segments_it>
-    f { segments, num_segments, (int)count, spacing, shift, p };
+    f { segments, num_segments, (int)count, spacing,
+      detail::int_divider_t::make(spacing), p };
+  cta_launch<nt>(f, div_up(num_segments, nt * vt), context);
+  return num_partitions;
+}
+
+// Same splits as pairs p[2 * i] = items, p[2 * i + 1] = segment starts in
+// front of split i, every inner split moved back to an item index that is a
+// multiple of `snap` where fewer than `window` starts have to move with it
+// (see lbs_partition_scatter_f).  2 * (div_up(count + num_segments, spacing)
+// + 1) ints.  Tiles cut this way hold at most spacing + snap + window - 2
+// merged elements.
+template<int snap, int window, typename segments_it>
+int load_balance_partitions_snapped(int count, segments_it segments,
+  int num_segments, int spacing, int* p, context_t& context) {
+  enum { nt = 256, vt = 4 };
+  int64_t total = (int64_t)count + num_segments;
+  int num_partitions = (int)div_up(total, (int64_t)spacing) + 1;
+  if(total >= ((int64_t)1 << 31))
+    throw cuda_exception_t(hipErrorInvalidValue);
+  if(!num_segments) {
+    // no starts: split i is (min(spacing * i, count) rounded down, 0).
+    transform<256>([=]MGPU_DEVICE(int index) {
+      int64_t d = (int64_t)spacing * index;
+      int a = d < count ? (int)(d - d % snap) : count;
+      p[2 * index] = a;
+      p[2 * index + 1] = 0;
+    }, num_partitions, context);
+    return num_partitions;
+  }
+  detail::lbs_partition_scatter_f<nt, int, segments_it, snap, window>
+    f { segments, num_segments, count, spacing,
+      detail::int_divider_t::make(spacing), p };
   cta_launch<nt>(f, div_up(num_segments, nt * vt), context);
   return num_partitions;
 }

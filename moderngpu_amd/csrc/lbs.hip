@@ -18,8 +18,9 @@ template<> struct bytes_type_t<4> { typedef uint32_t type; };
 template<> struct bytes_type_t<8> { typedef uint64_t type; };
 template<> struct bytes_type_t<16> { typedef bytes16_t type; };
 
-int partition_count(int count, int num_segments) {
-  return div_up(count + num_segments, mgpu_hip_lbs_tile_size()) + 1;
+size_t partition_ints(int count, int num_segments) {
+  return detail::lbs_partition_ints(count + num_segments,
+    lbs_launch_t::sm_ptx::nt * lbs_launch_t::sm_ptx::vt);
 }
 
 bool lbs_args_ok(int count, const int* segments, int num_segments,
@@ -131,7 +132,7 @@ extern "C" {
 size_t mgpu_hip_lbs_workspace_bytes(int count, int num_segments) {
   if(!sizes_ok(count, num_segments)) return 0;
   if(!(count + num_segments)) return 0;
-  return sizeof(int) * (size_t)partition_count(count, num_segments);
+  return sizeof(int) * partition_ints(count, num_segments);
 }
 
 int mgpu_hip_load_balance_search_phases(int count, const int* segments,

@@ -57,8 +57,8 @@ int mgpu_hip_segreduce_tile_size(int dtype) {
 }
 
 int mgpu_hip_lbs_tile_size(void) {
-  return detail::lbs_launch_default_t::sm_ptx::nt *
-    detail::lbs_launch_default_t::sm_ptx::vt;
+  return detail::lbs_tile_spacing(detail::lbs_launch_default_t::sm_ptx::nt *
+    detail::lbs_launch_default_t::sm_ptx::vt);
 }
 
 int mgpu_hip_partition_count(int64_t a_count, int64_t b_count,

@@ -52,8 +52,9 @@ def test_workspace_sizes():
     assert 0 < small < big < (1 << 22)
     assert L.mgpu_hip_segreduce_workspace_bytes(1 << 30, 1 << 30, 4) == 0  # index overflow
     assert L.mgpu_hip_segreduce_workspace_bytes(10, 10, 77) == 0           # bad dtype
+    # one (items, starts) pair of ints per tile split
     assert L.mgpu_hip_lbs_workspace_bytes(1 << 28, 1 << 24) == \
-        4 * (((1 << 28) + (1 << 24)) // m.lbs_tile_size() + 1)
+        8 * (((1 << 28) + (1 << 24)) // m.lbs_tile_size() + 1 + 1)
 
 
 def test_bad_arguments_are_rejected_without_a_gpu():
