@@ -48,25 +48,30 @@ namespace detail {
 // types use one (possibly unaligned) 16-byte global load; anything else is
 // element-wise through operator[].
 
+// load(input, base, offset, x) reads items base + offset + [0, W); base is
+// the same in all threads of the CTA and offset is not negative, which lets
+// a pointer input be addressed as (scalar base address, 32-bit lane offset).
 template<typename input_it, typename type_t, int W>
 struct tile_loader_t {
-  MGPU_DEVICE static void load(input_it input, int index, type_t (&x)[W]) {
+  MGPU_DEVICE static void load(input_it input, int base, unsigned offset,
+    type_t (&x)[W]) {
     PRAGMA_UNROLL
-    for(int e = 0; e < W; ++e) x[e] = input[index + e];
+    for(int e = 0; e < W; ++e) x[e] = input[base + (int)offset + e];
   }
 };
 
 template<typename type_t, int W>
 struct pointer_loader_t {
-  MGPU_DEVICE static void load(const type_t* input, int index,
-    type_t (&x)[W]) {
+  MGPU_DEVICE static void load(const type_t* input, int base,
+    unsigned offset, type_t (&x)[W]) {
+    const type_t* tile = input + base;
     if constexpr(W > 1) {
       typedef typename vec_t<type_t, W>::type_u v_t;
-      v_t v = *(const v_t*)(input + index);
+      v_t v = *(const v_t*)(tile + offset);
       PRAGMA_UNROLL
       for(int e = 0; e < W; ++e) x[e] = v[e];
     } else
-      x[0] = input[index];
+      x[0] = tile[offset];
   }
 };
 template<typename type_t, int W>
@@ -88,19 +93,19 @@ struct spmv_input_t {
 };
 template<typename type_t, int W>
 struct tile_loader_t<spmv_input_t<type_t>, type_t, W> {
-  MGPU_DEVICE static void load(spmv_input_t<type_t> in, int index,
-    type_t (&x)[W]) {
+  MGPU_DEVICE static void load(spmv_input_t<type_t> in, int base,
+    unsigned offset, type_t (&x)[W]) {
     type_t a[W];
     int c[W];
-    pointer_loader_t<type_t, W>::load(in.matrix, index, a);
+    pointer_loader_t<type_t, W>::load(in.matrix, base, offset, a);
     // Columns are 4-byte: W of them are 16 bytes or less.
     if constexpr(W > 1) {
       typedef typename vec_t<int, W>::type_u v_t;
-      v_t v = *(const v_t*)(in.columns + index);
+      v_t v = *(const v_t*)(in.columns + base + offset);
       PRAGMA_UNROLL
       for(int e = 0; e < W; ++e) c[e] = v[e];
     } else
-      c[0] = in.columns[index];
+      c[0] = in.columns[base + offset];
     PRAGMA_UNROLL
     for(int e = 0; e < W; ++e) x[e] = a[e] * in.vector[c[e]];
   }
@@ -110,19 +115,23 @@ struct tile_loader_t<spmv_input_t<type_t>, type_t, W> {
 // One step of the thread-serial segmented scan: the running fold `prev`
 // continues into `cur` unless bit i of `bits` marks a segment start at this
 // item.  The generic form is a compare and a select around op().  For the
-// built-in operators on 4/8-byte arithmetic types the select folds into bit
-// arithmetic (no compare, no SGPR mask round trip):
-//   plus:     cur + (prev with all bits cleared when a segment starts here)
-//   max/min:  op(start ? cur : prev, cur), the choice done with one
-//             bitfield-insert per 32-bit word; op(cur, cur) == cur.
+// built-in operators on 4/8-byte arithmetic types the select is done with bit
+// arithmetic on a mask spread from the flag bit (one v_bfe_i32; written as
+// inline assembly because the compiler otherwise turns the mask back into a
+// compare, a lane mask in SGPRs and a select):
+//   plus:     cur + (prev & keep), keep = all ones unless a segment starts
+//   max/min:  op(start ? cur : prev, cur) with one bitfield-insert per 32-bit
+//             word for the choice; op(cur, cur) == cur.
 // For floating-point plus a segment made only of -0.0 sums to +0.0; sums are
 // compared with a tolerance, and max/min stay bit-exact.
 
 template<typename op_t, typename type_t, typename enable_t = void>
 struct segscan_step_t {
-  MGPU_DEVICE static type_t step(type_t prev, type_t cur, unsigned bits,
-    int i, op_t op) {
-    return ((bits >> i) & 1) ? cur : op(prev, cur);
+  // nbits = complement of the start bits.
+  template<int i>
+  MGPU_DEVICE static type_t step(type_t prev, type_t cur, unsigned nbits,
+    op_t op) {
+    return ((nbits >> i) & 1) ? op(prev, cur) : cur;
   }
 };
 
@@ -137,10 +146,11 @@ struct bitwise_word_t {
     type_t x; __builtin_memcpy(&x, &y, sizeof(x)); return x;
   }
   // All ones if bit i of bits is set, else zero.
-  MGPU_DEVICE static type spread(unsigned bits, int i) {
-    // the builtin's result is declared unsigned: make it signed before
-    // widening so that the 64-bit mask is all ones, not 32 ones.
-    return (type)(long long)(int)__builtin_amdgcn_sbfe(bits, i, 1);
+  template<int i>
+  MGPU_DEVICE static type spread(unsigned bits) {
+    int m;
+    asm("v_bfe_i32 %0, %1, %2, 1" : "=v"(m) : "v"(bits), "n"(i));
+    return (type)(long long)m;
   }
 };
 
@@ -153,20 +163,22 @@ struct is_word_arithmetic_t {
 template<typename type_t>
 struct segscan_step_t<plus_t<type_t>, type_t,
   enable_if_t<is_word_arithmetic_t<type_t>::value> > {
-  MGPU_DEVICE static type_t step(type_t prev, type_t cur, unsigned bits,
-    int i, plus_t<type_t>) {
+  template<int i>
+  MGPU_DEVICE static type_t step(type_t prev, type_t cur, unsigned nbits,
+    plus_t<type_t>) {
     typedef bitwise_word_t<type_t> w;
-    return w::from(w::to(prev) & ~w::spread(bits, i)) + cur;
+    return w::from(w::to(prev) & w::template spread<i>(nbits)) + cur;
   }
 };
 
 template<typename op_t, typename type_t>
 struct segscan_select_step_t {
-  MGPU_DEVICE static type_t step(type_t prev, type_t cur, unsigned bits,
-    int i, op_t op) {
+  template<int i>
+  MGPU_DEVICE static type_t step(type_t prev, type_t cur, unsigned nbits,
+    op_t op) {
     typedef bitwise_word_t<type_t> w;
-    typename w::type m = w::spread(bits, i);
-    return op(w::from((m & w::to(cur)) | (~m & w::to(prev))), cur);
+    typename w::type keep = w::template spread<i>(nbits);
+    return op(w::from((keep & w::to(prev)) | (~keep & w::to(cur))), cur);
   }
 };
 template<typename type_t>
@@ -177,6 +189,22 @@ template<typename type_t>
 struct segscan_step_t<minimum_t<type_t>, type_t,
   enable_if_t<is_word_arithmetic_t<type_t>::value> > :
   segscan_select_step_t<minimum_t<type_t>, type_t> { };
+
+// x[i] = step<i>(x[i - 1], x[i]) for i = first .. vt - 1.
+template<int i, int vt>
+struct segscan_thread_t {
+  template<typename op_t, typename type_t>
+  MGPU_DEVICE static void run(type_t (&x)[vt], unsigned nbits, op_t op) {
+    x[i] = segscan_step_t<op_t, type_t>::template step<i>(x[i - 1], x[i],
+      nbits, op);
+    segscan_thread_t<i + 1, vt>::run(x, nbits, op);
+  }
+};
+template<int vt>
+struct segscan_thread_t<vt, vt> {
+  template<typename op_t, typename type_t>
+  MGPU_DEVICE static void run(type_t (&)[vt], unsigned, op_t) { }
+};
 
 ////////////////////////////////////////////////////////////////////////////////
 // Default tiles on gfx950: 256 threads x 16 values for 4- and 8-byte values
@@ -227,31 +255,48 @@ struct segreduce_tile_f {
   int* carry_codes;
   int num_tiles;
 
+  typedef typename launch_t::sm_ptx params_t;
+  enum {
+    nt = params_t::nt, vt = params_t::vt, nv = nt * vt,
+    W = chunk_width_t<type_t, vt>::value,
+    chunks = vt / W,
+    flag_words = nv / 32 + 2
+  };
+  static_assert(vt <= 32, "segreduce tiles hold at most 32 values/thread");
+  typedef tile_layout_t<W> layout_t;
+  typedef cta_segscan_t<nt, type_t> segscan_t;
+  typedef tile_loader_t<input_it, type_t, W> loader_t;
+
+  struct storage_t {
+    alignas(16) type_t values[layout_t::capacity(nv)];
+    type_t flow[nt];              // fold flowing into each thread
+    unsigned flags[flag_words];   // bit p: a segment starts at tile item p
+    typename segscan_t::storage_t segscan;
+  };
+
   MGPU_DEVICE void operator()(int tid, int cta) const {
     // Neighbouring tiles run on the same XCD (see xcd_tile).
     cta = xcd_tile(cta, num_tiles);
     if(cta >= num_tiles) return;
-    typedef typename launch_t::sm_ptx params_t;
-    enum {
-      nt = params_t::nt, vt = params_t::vt, nv = nt * vt,
-      W = chunk_width_t<type_t, vt>::value,
-      chunks = vt / W,
-      flag_words = nv / 32 + 2
-    };
-    static_assert(vt <= 32, "segreduce tiles hold at most 32 values/thread");
-    typedef tile_layout_t<W> layout_t;
-    typedef cta_segscan_t<nt, type_t> segscan_t;
-    typedef tile_loader_t<input_it, type_t, W> loader_t;
-
-    __shared__ struct {
-      alignas(16) type_t values[layout_t::capacity(nv)];
-      type_t flow[nt];              // fold flowing into each thread
-      unsigned flags[flag_words];   // bit p: a segment starts at tile item p
-      typename segscan_t::storage_t segscan;
-    } shared;
+    __shared__ storage_t shared;
 
     merge_range_t range = tile_range(count, num_segments, cta, nv,
       mp_data[cta], mp_data[cta + 1]);
+    // A tile that lies nv items or more in front of the end of the input
+    // reads nv items whatever its a_count is: what it reads past its own
+    // last item belongs to the next tile and is never looked at, and no
+    // load or LDS store needs a per-lane bounds check.  The kernel body
+    // exists once for such tiles and once with the checks.
+    if(range.a_begin <= count - nv)
+      tile(std::true_type(), tid, cta, range, shared);
+    else
+      tile(std::false_type(), tid, cta, range, shared);
+  }
+
+  template<typename interior_t>
+  MGPU_DEVICE void tile(interior_t, int tid, int cta, merge_range_t range,
+    storage_t& shared) const {
+    enum { interior = interior_t::value };
     int a_count = range.a_count();
     int b_count = range.b_count();
 
@@ -269,15 +314,22 @@ struct segreduce_tile_f {
     if(!tid && range.b_begin > 0) open_start = segments[range.b_begin - 1];
     // The item loads; they are consumed after the flag setup.
     type_t r[chunks][W];
-    PRAGMA_UNROLL
-    for(int i = 0; i < chunks; ++i) {
-      int p = W * (nt * i + tid);
-      if(p + W <= a_count)
-        loader_t::load(input, range.a_begin + p, r[i]);
-      else {
-        PRAGMA_UNROLL
-        for(int e = 0; e < W; ++e)
-          if(p + e < a_count) r[i][e] = input[range.a_begin + p + e];
+    if constexpr(interior) {
+      PRAGMA_UNROLL
+      for(int i = 0; i < chunks; ++i)
+        loader_t::load(input, range.a_begin, (unsigned)(W * (nt * i + tid)),
+          r[i]);
+    } else {
+      PRAGMA_UNROLL
+      for(int i = 0; i < chunks; ++i) {
+        int p = W * (nt * i + tid);
+        if(p + W <= a_count)
+          loader_t::load(input, range.a_begin, (unsigned)p, r[i]);
+        else {
+          PRAGMA_UNROLL
+          for(int e = 0; e < W; ++e)
+            if(p + e < a_count) r[i][e] = input[range.a_begin + p + e];
+        }
       }
     }
 
@@ -295,7 +347,7 @@ struct segreduce_tile_f {
     PRAGMA_UNROLL
     for(int i = 0; i < chunks; ++i) {
       int p = W * (nt * i + tid);
-      if(p < a_count)
+      if(interior || p < a_count)
         lds_store_chunk<W>(shared.values + layout_t::index(p), r[i]);
     }
     __syncthreads();
@@ -320,16 +372,14 @@ struct segreduce_tile_f {
     }
 
     // Inclusive segmented scan of the thread's items, left to right.
-    PRAGMA_UNROLL
-    for(int i = 1; i < vt; ++i)
-      x[i] = segscan_step_t<op_t, type_t>::step(x[i - 1], x[i], bits, i, op);
+    segscan_thread_t<1, vt>::run(x, ~bits, op);
 
     PRAGMA_UNROLL
     for(int c = 0; c < chunks; ++c) {
       type_t chunk[W];
       PRAGMA_UNROLL
       for(int e = 0; e < W; ++e) chunk[e] = x[W * c + e];
-      if(vt * tid + W * c < a_count)
+      if(interior || vt * tid + W * c < a_count)
         lds_store_chunk<W>(shared.values + layout_t::index(vt * tid + W * c),
           chunk);
     }

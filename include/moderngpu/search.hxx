@@ -102,7 +102,7 @@ struct int_divider_t {
 // 16-byte load, nothing dependent -- and writes the splits of the tile
 // boundaries that fall between a start and the next one: none for most
 // segments, one for a segment that straddles a boundary, many for a segment
-// that spans tiles (long runs are queued in LDS and written by the whole CTA).
+// that spans tiles (long runs are written by the whole wavefront).
 //
 // With snap > 0 the kernel writes pairs (a, b) = (items, starts) in front of
 // each split instead of a alone, and moves every split except the first and
@@ -146,11 +146,6 @@ struct lbs_partition_scatter_f {
   }
 
   MGPU_DEVICE void operator()(int tid, int cta) const {
-    __shared__ int queue_size;
-    __shared__ int queue[nt * vt][3];     // first boundary, how many, j + 1
-    if(!tid) queue_size = 0;
-    __syncthreads();
-
     int total = count + num_segments;
     int j0 = vt * (nt * cta + tid);
 
@@ -222,23 +217,35 @@ struct lbs_partition_scatter_f {
       } else if(n > 0)
         write_inside(first, j + 1);
 
-      if(n > 1) {
-        if(n <= direct) {
-          for(int k = 1; k < n; ++k) write_inside(first + k, j + 1);
-        } else {
-          int slot = atomicAdd(&queue_size, 1);
-          queue[slot][0] = first + 1;
-          queue[slot][1] = n - 1;
-          queue[slot][2] = j + 1;
-        }
+      // The other splits inside segment j: written by the thread itself when
+      // there are few, by the whole wavefront when the segment spans many
+      // tiles.
+      if(n > 1 && n <= direct)
+        for(int k = 1; k < n; ++k) write_inside(first + k, j + 1);
+      lanemask_t spanning = ballot(n > direct);
+      while(spanning) {
+        int src = (int)__builtin_ctzll(spanning);
+        spanning &= spanning - 1;
+        int src_first = readlane(first, src);
+        int src_n = readlane(n, src);
+        int src_before = readlane(j, src) + 1;
+        if constexpr(snap == 0 && std::is_same<int_t, int>::value) {
+          // four consecutive splits per lane and 16-byte store.
+          typedef int v4_t __attribute__((ext_vector_type(4), aligned(4)));
+          for(int k = 1 + 4 * lane; k < src_n; k += 4 * warp_size) {
+            int base = (src_first + k) * spacing - src_before;
+            if(k + 4 <= src_n) {
+              v4_t v = { base, base + spacing, base + 2 * spacing,
+                base + 3 * spacing };
+              *(v4_t*)(p + src_first + k) = v;
+            } else
+              for(int i = 0; k + i < src_n; ++i)
+                p[src_first + k + i] = base + i * spacing;
+          }
+        } else
+          for(int k = 1 + lane; k < src_n; k += warp_size)
+            write_inside(src_first + k, src_before);
       }
-    }
-    __syncthreads();
-
-    int queued = queue_size;
-    for(int q = 0; q < queued; ++q) {
-      int first = queue[q][0], n = queue[q][1], before = queue[q][2];
-      for(int k = tid; k < n; k += nt) write_inside(first + k, before);
     }
 
     if(!cta && !tid) {
