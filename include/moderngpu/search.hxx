@@ -98,8 +98,8 @@ struct int_divider_t {
 // position m_j = segments[j] + j (all items before it plus all starts before
 // it), so the split of cross-diagonal d is d - #{j : m_j < d}.  Instead of
 // one binary search per split (log2(num_segments) dependent, scattered
-// loads each) every thread reads four consecutive segment starts -- one
-// 16-byte load, nothing dependent -- and writes the splits of the tile
+// loads each) every thread reads vt consecutive segment starts -- 16-byte
+// loads, nothing dependent -- and writes the splits of the tile
 // boundaries that fall between a start and the next one: none for most
 // segments, one for a segment that straddles a boundary, many for a segment
 // that spans tiles (long runs are written by the whole wavefront).
@@ -113,9 +113,10 @@ struct int_divider_t {
 // them the split stays where it is.  A moved split retreats by at most
 // (snap - 1) + (window - 1) merged elements.
 template<int nt, typename int_t, typename segments_it, int snap = 0,
-  int window = 32>
+  int window = 32, int vt_ = 8>
 struct lbs_partition_scatter_f {
-  enum { vt = 4, direct = 8 };
+  enum { vt = vt_, direct = 8 };
+  static_assert(0 == vt % 4, "segments are read four at a time");
   segments_it segments;
   int num_segments;
   int count;
@@ -155,8 +156,12 @@ struct lbs_partition_scatter_f {
     if(j0 + vt < num_segments) {
       if constexpr(std::is_pointer<segments_it>::value) {
         typedef int v4_t __attribute__((ext_vector_type(4), aligned(4)));
-        v4_t v = *(const v4_t*)(segments + j0);
-        starts[0] = v[0]; starts[1] = v[1]; starts[2] = v[2]; starts[3] = v[3];
+        PRAGMA_UNROLL
+        for(int q = 0; q < vt / 4; ++q) {
+          v4_t v = *(const v4_t*)(segments + j0 + 4 * q);
+          starts[4 * q] = v[0]; starts[4 * q + 1] = v[1];
+          starts[4 * q + 2] = v[2]; starts[4 * q + 3] = v[3];
+        }
       } else {
         PRAGMA_UNROLL
         for(int e = 0; e < vt; ++e) starts[e] = segments[j0 + e];
@@ -284,7 +289,7 @@ int merge_path_partitions_into(a_keys_it a, int64_t a_count, b_keys_it b,
 template<typename segments_it, typename int_t>
 int load_balance_partitions_into(int64_t count, segments_it segments,
   int num_segments, int spacing, int_t* p, context_t& context) {
-  enum { nt = 256, vt = 4 };
+  enum { nt = 256, vt = 8 };
   int num_partitions = (int)div_up(count + num_segments, (int64_t)spacing) + 1;
   if(count + num_segments >= ((int64_t)1 << 31))
     throw cuda_exception_t(hipErrorInvalidValue);
@@ -292,7 +297,7 @@ int load_balance_partitions_into(int64_t count, segments_it segments,
     return merge_path_partitions_into<bounds_upper>(
       counting_iterator_t<int_t>(0), count, segments, (int64_t)0,
       (int64_t)spacing, less_t<int_t>(), p, context);
-  detail::lbs_partition_scatter_f<nt, int_t, segments_it>
+  detail::lbs_partition_scatter_f<nt, int_t, segments_it, 0, 32, vt>
     f { segments, num_segments, (int)count, spacing,
       detail::int_divider_t::make(spacing), p };
   cta_launch<nt>(f, div_up(num_segments, nt * vt), context);
@@ -308,7 +313,7 @@ int load_balance_partitions_into(int64_t count, segments_it segments,
 template<int snap, int window, typename segments_it>
 int load_balance_partitions_snapped(int count, segments_it segments,
   int num_segments, int spacing, int* p, context_t& context) {
-  enum { nt = 256, vt = 4 };
+  enum { nt = 256, vt = 8 };
   int64_t total = (int64_t)count + num_segments;
   int num_partitions = (int)div_up(total, (int64_t)spacing) + 1;
   if(total >= ((int64_t)1 << 31))
@@ -323,7 +328,7 @@ int load_balance_partitions_snapped(int count, segments_it segments,
     }, num_partitions, context);
     return num_partitions;
   }
-  detail::lbs_partition_scatter_f<nt, int, segments_it, snap, window>
+  detail::lbs_partition_scatter_f<nt, int, segments_it, snap, window, vt>
     f { segments, num_segments, count, spacing,
       detail::int_divider_t::make(spacing), p };
   cta_launch<nt>(f, div_up(num_segments, nt * vt), context);
