@@ -239,7 +239,56 @@ def make_c1(copies):
     return wk
 
 
+def make_scan(copies, kind):
+    """The step in front of the path: 2^26 int32 segment lengths -> starts
+    (exclusive plus-scan), or the fold of 2^26 floats (reduce)."""
+    import torch
+    import moderngpu_amd as m
+    from oracle import oracle
+    n = 1 << 26
+    rng = np.random.Generator(np.random.PCG64(42))
+    wk = Workload()
+    wk.items = n
+    if kind == "scan":
+        host = rng.integers(0, 128, size=n, dtype=np.int32)
+        vals = [_dev(host)] + [torch.randint(0, 128, (n,), dtype=torch.int32, device="cuda")
+                               for _ in range(copies - 1)]
+        outs = [torch.empty(n, dtype=torch.int32, device="cuda") for _ in range(copies)]
+        red = torch.zeros(1, dtype=torch.int32, device="cuda")
+        wk.key, wk.dtype = "scan_i32", "i32"
+        wk.name = "exclusive plus-scan, 2^26 int32 (segment lengths -> starts)"
+        wk.bytes = n * 4 + n * 4
+        wk.kernel = "scan upsweep + spine + downsweep (whole call)"
+        wk.step = lambda i: m.scan(vals[i % copies], "plus", out=outs[i % copies],
+                                   reduction=red)[0]
+        wk.tiles = wk.step
+        wk.check = lambda: bool(np.array_equal(
+            wk.step(0).cpu().numpy(), oracle.scan(host, "plus", 0, inclusive=False)[0]))
+        wk.cpu = lambda: (lambda: oracle.scan(host, "plus", 0, inclusive=False))
+    else:
+        host = rng.random(n, dtype=np.float32)
+        vals = [_dev(host)] + [torch.rand(n, dtype=torch.float32, device="cuda")
+                               for _ in range(copies - 1)]
+        out = torch.zeros(1, dtype=torch.float32, device="cuda")
+        wk.key, wk.dtype = "reduce_f32", "f32"
+        wk.name = "plus-reduce, 2^26 float32"
+        wk.bytes = n * 4
+        wk.kernel = "scan_upsweep_f + reduce_final_f (whole call)"
+        wk.step = lambda i: m.reduce(vals[i % copies], "plus", out=out)
+        wk.tiles = wk.step
+
+        def check():
+            got = float(wk.step(0).item())
+            exact = float(np.sum(host.astype(np.float64)))
+            return abs(got - exact) <= 1e-5 * exact
+        wk.check = check
+        wk.cpu = lambda: (lambda: oracle.scan(host, "plus", 0, inclusive=True))
+    return wk
+
+
 FACTORIES = {
+    "scan_i32": lambda c: make_scan(c, "scan"),
+    "reduce_f32": lambda c: make_scan(c, "reduce"),
     "c1_segreduce_i32": make_c1,
     "c2_segreduce_f32": make_c2,
     "c3_load_balance_search": lambda c: make_c3(c, False),

@@ -115,6 +115,17 @@ MGPU_HIP_API int mgpu_hip_transform_segreduce_mod13(int count,
   const int* segments, int num_segments, int* output, int init,
   void* workspace, size_t workspace_bytes, mgpu_stream_t stream);
 
+/* mgpu::lbs_segreduce (kernel_segreduce.hxx:303-404) with the functor of the
+ * reference's own test, f(index, seg, rank) = seg + rank, int32 plus
+ * (tests/test_segreduce.cu:11-13, :29-30): output[s] = sum over the items of
+ * segment s of (s + rank), init for empty segments.  Shows the computed-items
+ * path through the C ABI; arbitrary functors and cached iterators need the
+ * C++ templates.  Workspace: mgpu_hip_segreduce_workspace_bytes(count,
+ * num_segments, MGPU_I32). */
+MGPU_HIP_API int mgpu_hip_lbs_segreduce_seg_plus_rank(int count,
+  const int* segments, int num_segments, int* output, int init,
+  void* workspace, size_t workspace_bytes, mgpu_stream_t stream);
+
 /* mgpu::spmv (kernel_segreduce.hxx:285-298): CSR y = A * x.
  * output[r] = sum over the row's nonzeros k of matrix[k] * vector[columns[k]];
  * segments = row starts (num_segments rows, no trailing nnz entry);
@@ -179,6 +190,32 @@ MGPU_HIP_API int mgpu_hip_interval_move(const void* input, int elem_bytes,
   int count, const int* segments, int num_segments, const int* scatter,
   const int* gather, void* output, void* workspace, size_t workspace_bytes,
   mgpu_stream_t stream);
+
+/* ---- scan and reduce (the steps on either side of the path) ------------- */
+
+/* Bytes of workspace mgpu_hip_scan needs for `count` items of `dtype`. */
+MGPU_HIP_API size_t mgpu_hip_scan_workspace_bytes(int count, int dtype);
+
+/* mgpu::scan / scan_event (kernel_scan.hxx:11-165) for pointer inputs.
+ * inclusive == 0: output[0] = 0 and output[i] = input[0] op ... op
+ * input[i - 1]; inclusive != 0: output[i] = input[0] op ... op input[i].
+ * The zero is only placed, never folded (so an exclusive maximum scan of
+ * negative values still starts with 0, as in the reference).  The fold of all
+ * items is stored to *reduction when reduction is not NULL (device memory, or
+ * host memory the device can write); for count == 0 that is 0.  input may
+ * equal output. */
+MGPU_HIP_API int mgpu_hip_scan(const void* input, int count, void* output,
+  int dtype, int op, int inclusive, void* reduction, void* workspace,
+  size_t workspace_bytes, mgpu_stream_t stream);
+
+/* Bytes of workspace mgpu_hip_reduce needs. */
+MGPU_HIP_API size_t mgpu_hip_reduce_workspace_bytes(int count, int dtype);
+
+/* mgpu::reduce (kernel_reduce.hxx:11-57) for pointer inputs: *reduction =
+ * input[0] op ... op input[count - 1]; nothing is stored for count == 0. */
+MGPU_HIP_API int mgpu_hip_reduce(const void* input, int count,
+  void* reduction, int dtype, int op, void* workspace,
+  size_t workspace_bytes, mgpu_stream_t stream);
 
 #ifdef __cplusplus
 }

@@ -169,6 +169,59 @@ MGPU_DEVICE inline void lds_store_chunk(type_t* p, const type_t (&x)[W]) {
     p[0] = x[0];
 }
 
+// Loading W consecutive tile items.  Raw pointers to 4/8-byte arithmetic
+// types use one (possibly unaligned) 16-byte global load; anything else is
+// element-wise through operator[].
+
+// load(input, base, offset, x) reads items base + offset + [0, W); base is
+// the same in all threads of the CTA and offset is not negative, which lets
+// a pointer input be addressed as (scalar base address, 32-bit lane offset).
+template<typename input_it, typename type_t, int W>
+struct tile_loader_t {
+  MGPU_DEVICE static void load(input_it input, int base, unsigned offset,
+    type_t (&x)[W]) {
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) x[e] = input[base + (int)offset + e];
+  }
+};
+
+template<typename type_t, int W>
+struct pointer_loader_t {
+  MGPU_DEVICE static void load(const type_t* input, int base,
+    unsigned offset, type_t (&x)[W]) {
+    const type_t* tile = input + base;
+    if constexpr(W > 1) {
+      typedef typename vec_t<type_t, W>::type_u v_t;
+      v_t v = *(const v_t*)(tile + offset);
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) x[e] = v[e];
+    } else
+      x[0] = tile[offset];
+  }
+};
+template<typename type_t, int W>
+struct tile_loader_t<const type_t*, type_t, W> : pointer_loader_t<type_t, W> { };
+template<typename type_t, int W>
+struct tile_loader_t<type_t*, type_t, W> : pointer_loader_t<type_t, W> { };
+
+// Stores W consecutive elements.  Element types whose size is a multiple of
+// four bytes go out as 16-byte stores (global_store_dwordx4 only needs dword
+// alignment); smaller ones element by element.
+template<int W, typename type_t>
+MGPU_DEVICE inline void store_consecutive(type_t* dest,
+  const type_t (&x)[W]) {
+  if constexpr(0 == sizeof(type_t) % 4 && W * sizeof(type_t) <= 64) {
+    enum { words = W * sizeof(type_t) / 4 };
+    typedef unsigned v_t __attribute__((ext_vector_type(words), aligned(4)));
+    v_t v;
+    __builtin_memcpy(&v, x, sizeof(v));
+    *(v_t*)dest = v;
+  } else {
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) dest[e] = x[e];
+  }
+}
+
 } // namespace detail
 
 ////////////////////////////////////////////////////////////////////////////////

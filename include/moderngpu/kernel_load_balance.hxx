@@ -36,24 +36,6 @@ struct is_chunk_functor_t<func_t,
   typename std::conditional<false, typename func_t::chunk_functor_tag,
     void>::type> : std::true_type { };
 
-// Stores W consecutive elements.  Element types whose size is a multiple of
-// four bytes go out as 16-byte stores (global_store_dwordx4 only needs dword
-// alignment); smaller ones element by element.
-template<int W, typename type_t>
-MGPU_DEVICE inline void store_consecutive(type_t* dest,
-  const type_t (&x)[W]) {
-  if constexpr(0 == sizeof(type_t) % 4 && W * sizeof(type_t) <= 64) {
-    enum { words = W * sizeof(type_t) / 4 };
-    typedef unsigned v_t __attribute__((ext_vector_type(words), aligned(4)));
-    v_t v;
-    __builtin_memcpy(&v, x, sizeof(v));
-    *(v_t*)dest = v;
-  } else {
-    PRAGMA_UNROLL
-    for(int e = 0; e < W; ++e) dest[e] = x[e];
-  }
-}
-
 template<typename launch_t, typename func_t, typename segments_it,
   typename pointers_t, typename int_t>
 struct transform_lbs_f {

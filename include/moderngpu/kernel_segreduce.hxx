@@ -44,41 +44,6 @@ BEGIN_MGPU_NAMESPACE
 namespace detail {
 
 ////////////////////////////////////////////////////////////////////////////////
-// Loading W consecutive tile items.  Raw pointers to 4/8-byte arithmetic
-// types use one (possibly unaligned) 16-byte global load; anything else is
-// element-wise through operator[].
-
-// load(input, base, offset, x) reads items base + offset + [0, W); base is
-// the same in all threads of the CTA and offset is not negative, which lets
-// a pointer input be addressed as (scalar base address, 32-bit lane offset).
-template<typename input_it, typename type_t, int W>
-struct tile_loader_t {
-  MGPU_DEVICE static void load(input_it input, int base, unsigned offset,
-    type_t (&x)[W]) {
-    PRAGMA_UNROLL
-    for(int e = 0; e < W; ++e) x[e] = input[base + (int)offset + e];
-  }
-};
-
-template<typename type_t, int W>
-struct pointer_loader_t {
-  MGPU_DEVICE static void load(const type_t* input, int base,
-    unsigned offset, type_t (&x)[W]) {
-    const type_t* tile = input + base;
-    if constexpr(W > 1) {
-      typedef typename vec_t<type_t, W>::type_u v_t;
-      v_t v = *(const v_t*)(tile + offset);
-      PRAGMA_UNROLL
-      for(int e = 0; e < W; ++e) x[e] = v[e];
-    } else
-      x[0] = tile[offset];
-  }
-};
-template<typename type_t, int W>
-struct tile_loader_t<const type_t*, type_t, W> : pointer_loader_t<type_t, W> { };
-template<typename type_t, int W>
-struct tile_loader_t<type_t*, type_t, W> : pointer_loader_t<type_t, W> { };
-
 // The fused spmv load: matrix[k] * vector[columns[k]], with the matrix values
 // and column indices of W consecutive nonzeros fetched as 16-byte loads.
 template<typename type_t>
@@ -238,6 +203,41 @@ struct carry_code_t {
 };
 
 ////////////////////////////////////////////////////////////////////////////////
+// Items that are not read but computed per (index, segment, rank): the input
+// of lbs_segreduce.  The tile kernel runs the load-balancing search of the
+// tile first -- its LDS is handed back before the reduction needs any -- and
+// calls f(index, seg, rank, cached values, args...) for every item of the
+// tile.
+
+template<typename func_t, typename pointers_t, typename type_t>
+struct lbs_input_t {
+  typedef type_t value_type;
+  func_t f;
+  pointers_t caching_iterators;
+};
+
+template<typename input_it>
+struct is_lbs_input_t : std::false_type { };
+template<typename func_t, typename pointers_t, typename type_t>
+struct is_lbs_input_t<lbs_input_t<func_t, pointers_t, type_t> > :
+  std::true_type { };
+
+// LDS the item source needs while it produces a tile's items.
+template<typename input_it, int nt, int vt>
+struct tile_source_storage_t {
+  typedef empty_t type;
+};
+template<typename func_t, typename pointers_t, typename type_t, int nt,
+  int vt>
+struct tile_source_storage_t<lbs_input_t<func_t, pointers_t, type_t>, nt,
+  vt> {
+  struct type {
+    typename cta_load_balance_t<nt, vt>::storage_t lbs;
+    typename cached_segment_load_t<nt, pointers_t>::storage_t cached;
+  };
+};
+
+////////////////////////////////////////////////////////////////////////////////
 // K2
 
 template<typename launch_t, typename input_it, typename segments_it,
@@ -267,14 +267,21 @@ struct segreduce_tile_f {
   typedef cta_segscan_t<nt, type_t> segscan_t;
   typedef tile_loader_t<input_it, type_t, W> loader_t;
 
-  struct storage_t {
+  struct work_storage_t {
     alignas(16) type_t values[layout_t::capacity(nv)];
     type_t flow[nt];              // fold flowing into each thread
     unsigned flags[flag_words];   // bit p: a segment starts at tile item p
     typename segscan_t::storage_t segscan;
   };
+  // What produces the items may use the same LDS before the reduction does.
+  union storage_t {
+    work_storage_t work;
+    typename tile_source_storage_t<input_it, nt, vt>::type source;
+    MGPU_DEVICE storage_t() { }     // members may have constructors
+  };
 
-  MGPU_DEVICE void operator()(int tid, int cta) const {
+  template<typename... args_t>
+  MGPU_DEVICE void operator()(int tid, int cta, args_t... args) const {
     // Neighbouring tiles run on the same XCD (see xcd_tile).
     cta = xcd_tile(cta, num_tiles);
     if(cta >= num_tiles) return;
@@ -287,16 +294,55 @@ struct segreduce_tile_f {
     // last item belongs to the next tile and is never looked at, and no
     // load or LDS store needs a per-lane bounds check.  The kernel body
     // exists once for such tiles and once with the checks.
-    if(range.a_begin <= count - nv)
-      tile(std::true_type(), tid, cta, range, shared);
+    // Computed items exist for the tile's own index range only.
+    if(!is_lbs_input_t<input_it>::value && range.a_begin <= count - nv)
+      tile(std::true_type(), tid, cta, range, shared, args...);
     else
-      tile(std::false_type(), tid, cta, range, shared);
+      tile(std::false_type(), tid, cta, range, shared, args...);
   }
 
-  template<typename interior_t>
+  // The items of a tile computed from its load-balancing search, in the
+  // strided chunk order the reduction expects.
+  template<typename... args_t>
+  MGPU_DEVICE void compute_items(merge_range_t range, int tid,
+    type_t (&r)[chunks][W], storage_t& shared, args_t... args) const {
+    if constexpr(is_lbs_input_t<input_it>::value) {
+      typedef cta_load_balance_t<nt, vt> load_balance_t;
+      typedef typename load_balance_t::layout_t slot_layout_t;
+      typedef decltype(input.caching_iterators) pointers_t;
+      typedef cached_segment_load_t<nt, pointers_t> cached_load_t;
+      int a_count = range.a_count();
+      int seg_base = range.b_begin - 1;
+      load_balance_t().fill(range, segments, tid, shared.source.lbs);
+      const int* slots = shared.source.lbs.indices;
+      const int* starts = slots + load_balance_t::starts_offset(a_count);
+      bool staged = cached_load_t::stage(tid, seg_base, range.b_count() + 1,
+        shared.source.cached, input.caching_iterators);
+      PRAGMA_UNROLL
+      for(int i = 0; i < chunks; ++i) {
+        PRAGMA_UNROLL
+        for(int e = 0; e < W; ++e) {
+          int p = W * (nt * i + tid) + e;
+          if(p < a_count) {
+            int rel = slots[slot_layout_t::index(p)];
+            int seg = seg_base + rel;
+            int index = range.a_begin + p;
+            r[i][e] = input.f(index, seg, index - starts[rel],
+              cached_load_t::get(staged, rel, seg, shared.source.cached,
+                input.caching_iterators), args...);
+          }
+        }
+      }
+      // The search's LDS is about to hold the values.
+      __syncthreads();
+    }
+  }
+
+  template<typename interior_t, typename... args_t>
   MGPU_DEVICE void tile(interior_t, int tid, int cta, merge_range_t range,
-    storage_t& shared) const {
+    storage_t& storage, args_t... args) const {
     enum { interior = interior_t::value };
+    work_storage_t& shared = storage.work;
     int a_count = range.a_count();
     int b_count = range.b_count();
 
@@ -314,7 +360,9 @@ struct segreduce_tile_f {
     if(!tid && range.b_begin > 0) open_start = segments[range.b_begin - 1];
     // The item loads; they are consumed after the flag setup.
     type_t r[chunks][W];
-    if constexpr(interior) {
+    if constexpr(is_lbs_input_t<input_it>::value) {
+      compute_items(range, tid, r, storage, args...);
+    } else if constexpr(interior) {
       PRAGMA_UNROLL
       for(int i = 0; i < chunks; ++i)
         loader_t::load(input, range.a_begin, (unsigned)(W * (nt * i + tid)),
@@ -568,11 +616,11 @@ enum {
 // selects a subset for measurement; a later phase then relies on what an
 // earlier full call left in the workspace.
 template<typename launch_t, typename input_it, typename segments_it,
-  typename output_it, typename op_t, typename type_t>
+  typename output_it, typename op_t, typename type_t, typename... args_t>
 void segreduce_launch(input_it input, int count, segments_it segments,
   int num_segments, output_it output, op_t op, type_t init, void* workspace,
   const segreduce_workspace_t& ws, context_t& context,
-  int phases = phase_all) {
+  int phases = phase_all, args_t... args) {
 
   if(!ws.num_ctas) return;
   cta_dim_t cta_dim = launch_t::cta_dim(context);
@@ -589,7 +637,7 @@ void segreduce_launch(input_it input, int count, segments_it segments,
     segreduce_tile_f<launch_t, input_it, segments_it, output_it, op_t, type_t>
       k_reduce { input, count, segments, num_segments, output, op, init,
         mp_data, carry_values, carry_codes, ws.num_ctas };
-    cta_launch<launch_t>(k_reduce, xcd_grid(ws.num_ctas), context);
+    cta_launch<launch_t>(k_reduce, xcd_grid(ws.num_ctas), context, args...);
   }
 
   if((phases & phase_spine) && ws.num_ctas > 1) {
@@ -683,6 +731,52 @@ void transform_segreduce(func_t f, int count, segments_it segments,
 
   segreduce<launch_arg_t>(make_load_iterator<type_t>(f), count, segments,
     num_segments, output, op, init, context);
+}
+
+// Segmented reduction over computed items: output[s] = fold over the items i
+// of segment s of f(i, s, i - segments[s], cached values of s, args...);
+// empty segments get init.  caching_iterators is a tuple of iterators indexed
+// by segment, dereferenced once per segment and tile rather than per item
+// (interface after src/moderngpu/kernel_segreduce.hxx:303-404).
+template<typename launch_arg_t = empty_t, typename func_t,
+  typename segments_it, typename pointers_t, typename output_it,
+  typename op_t, typename type_t, typename... args_t>
+void lbs_segreduce(func_t f, int count, segments_it segments,
+  int num_segments, pointers_t caching_iterators, output_it output, op_t op,
+  type_t init, context_t& context, args_t... args) {
+
+  typedef typename conditional_typedef_t<launch_arg_t,
+    typename detail::segreduce_launch_default_t<type_t>::type_t_
+  >::type_t launch_t;
+
+  cta_dim_t cta_dim = launch_t::cta_dim(context);
+  detail::segreduce_workspace_t ws(count, num_segments, cta_dim.nv(),
+    sizeof(type_t));
+  if(!ws.num_ctas) return;
+
+  mem_t<char> workspace(ws.bytes, context);
+  detail::lbs_input_t<func_t, pointers_t, type_t>
+    input { f, caching_iterators };
+  detail::segreduce_launch<launch_t>(input, count, segments, num_segments,
+    output, op, init, workspace.data(), ws, context, detail::phase_all,
+    args...);
+}
+
+// Without cached values: f(index, seg, rank, args...).
+template<typename launch_arg_t = empty_t, typename func_t,
+  typename segments_it, typename output_it, typename op_t, typename type_t,
+  typename... args_t>
+void lbs_segreduce(func_t f, int count, segments_it segments,
+  int num_segments, output_it output, op_t op, type_t init,
+  context_t& context, args_t... args) {
+
+  lbs_segreduce<launch_arg_t>(
+    [=]MGPU_DEVICE(int index, int seg, int rank, tuple<>, args_t... args) {
+      return f(index, seg, rank, args...);
+    },
+    count, segments, num_segments, tuple<>(), output, op, init, context,
+    args...
+  );
 }
 
 // CSR sparse matrix * dense vector.  segments = row starts (num_segments

@@ -22,6 +22,7 @@ SIGNATURES = {
     "mgpu_hip_segreduce": (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_int, c_vp, c_vp, c_size, c_vp]),
     "mgpu_hip_segreduce_phases": (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_int, c_vp, c_vp, c_size, c_vp, c_int]),
     "mgpu_hip_transform_segreduce_mod13": (c_int, [c_int, c_vp, c_int, c_vp, c_int, c_vp, c_size, c_vp]),
+    "mgpu_hip_lbs_segreduce_seg_plus_rank": (c_int, [c_int, c_vp, c_int, c_vp, c_int, c_vp, c_size, c_vp]),
     "mgpu_hip_spmv": (c_int, [c_vp, c_vp, c_vp, c_int, c_vp, c_int, c_vp, c_int, c_vp, c_size, c_vp]),
     "mgpu_hip_spmv_phases": (c_int, [c_vp, c_vp, c_vp, c_int, c_vp, c_int, c_vp, c_int, c_vp, c_size, c_vp, c_int]),
     "mgpu_hip_lbs_workspace_bytes": (c_size, [c_int, c_int]),
@@ -33,6 +34,10 @@ SIGNATURES = {
     "mgpu_hip_interval_gather": (c_int, [c_vp, c_int, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_size, c_vp]),
     "mgpu_hip_interval_scatter": (c_int, [c_vp, c_int, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_size, c_vp]),
     "mgpu_hip_interval_move": (c_int, [c_vp, c_int, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_size, c_vp]),
+    "mgpu_hip_scan_workspace_bytes": (c_size, [c_int, c_int]),
+    "mgpu_hip_scan": (c_int, [c_vp, c_int, c_vp, c_int, c_int, c_int, c_vp, c_vp, c_size, c_vp]),
+    "mgpu_hip_reduce_workspace_bytes": (c_size, [c_int, c_int]),
+    "mgpu_hip_reduce": (c_int, [c_vp, c_int, c_vp, c_int, c_int, c_vp, c_size, c_vp]),
 }
 
 _lib = None

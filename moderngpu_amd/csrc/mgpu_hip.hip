@@ -32,6 +32,11 @@ int spmv_typed(const type_t* matrix, const int* columns, const type_t* vector,
   });
 }
 
+struct seg_plus_rank_f {
+  MGPU_DEVICE int operator()(int, int seg, int rank, tuple<>) const {
+    return seg + rank;
+  }
+};
 struct mod13_f {
   MGPU_DEVICE int operator()(int index) const { return index % 13; }
 };
@@ -181,6 +186,27 @@ int mgpu_hip_transform_segreduce_mod13(int count, const int* segments,
     detail::segreduce_launch<launch_t>(make_load_iterator<int>(mod13_f()),
       count, segments, num_segments, output, plus_t<int>(), init, workspace,
       ws, context);
+  });
+}
+
+int mgpu_hip_lbs_segreduce_seg_plus_rank(int count, const int* segments,
+  int num_segments, int* output, int init, void* workspace,
+  size_t workspace_bytes, mgpu_stream_t stream) {
+  if(!sizes_ok(count, num_segments) ||
+    (num_segments && (!segments || !output)))
+    return (int)hipErrorInvalidValue;
+  size_t need = mgpu_hip_segreduce_workspace_bytes(count, num_segments,
+    MGPU_I32);
+  if(need && (!workspace || workspace_bytes < need))
+    return (int)hipErrorInvalidValue;
+  typedef segreduce_launch_t<int>::type launch_t;
+  return guarded(stream, [&](context_t& context) {
+    detail::segreduce_workspace_t ws(count, num_segments,
+      launch_t::nv(context), sizeof(int));
+    detail::lbs_input_t<seg_plus_rank_f, tuple<>, int>
+      input { seg_plus_rank_f(), tuple<>() };
+    detail::segreduce_launch<launch_t>(input, count, segments, num_segments,
+      output, plus_t<int>(), init, workspace, ws, context);
   });
 }
 

@@ -117,6 +117,20 @@ def transform_segreduce_mod13(count, segments, init=-1, out=None):
     return out
 
 
+def lbs_segreduce_seg_plus_rank(count, segments, init=-1, out=None):
+    """lbs_segreduce with f(index, seg, rank) = seg + rank, int32 plus."""
+    _dev_i32(segments, "segments")
+    nseg = segments.numel()
+    if out is None:
+        out = torch.empty(nseg, dtype=torch.int32, device=segments.device)
+    need = lib().mgpu_hip_segreduce_workspace_bytes(count, nseg, 0)
+    ws = _workspace(need, segments.device)
+    _check(lib().mgpu_hip_lbs_segreduce_seg_plus_rank(
+        count, _ptr(segments), nseg, _ptr(out), init, _ptr(ws), ws.numel(),
+        _stream()))
+    return out
+
+
 def spmv(matrix, columns, vector, segments, out=None, phases=7, workspace=None):
     """CSR y = A x; segments are the row starts (no trailing nnz entry)."""
     _dev_i32(segments, "segments")
@@ -249,4 +263,45 @@ def binary_search_partitions(keys, count, spacing, bounds="lower"):
     _check(lib().mgpu_hip_binary_search_partitions(
         _ptr(keys), count, keys.numel(), spacing,
         1 if bounds == "upper" else 0, _ptr(out), _stream()))
+    return out
+
+
+def scan(values, op="plus", inclusive=False, out=None, reduction=None,
+         unsigned=False):
+    """Device-wide scan (mgpu::scan).  Exclusive: out[0] = 0, out[i] = fold of
+    values[:i]; inclusive: out[i] = fold of values[:i + 1].  The zero is only
+    placed, never folded.  ``reduction`` is an optional 1-element tensor (device
+    or pinned host memory) that receives the fold of everything; the returned
+    pair is (out, reduction)."""
+    if not values.is_cuda or not values.is_contiguous():
+        raise TypeError("values must be a contiguous CUDA tensor")
+    code = _dtype_code(values, unsigned)
+    count = values.numel()
+    if out is None:
+        out = torch.empty_like(values)
+    if reduction is not None and (reduction.dtype != values.dtype or reduction.numel() != 1):
+        raise TypeError("reduction must be one element of the values' type")
+    need = lib().mgpu_hip_scan_workspace_bytes(count, code)
+    ws = _workspace(need, values.device)
+    red = ctypes.c_void_p(reduction.data_ptr()) if reduction is not None else None
+    _check(lib().mgpu_hip_scan(
+        _ptr(values), count, _ptr(out), code, OPS[op], int(bool(inclusive)), red,
+        _ptr(ws), ws.numel(), _stream()))
+    return out, reduction
+
+
+def reduce(values, op="plus", out=None, unsigned=False):
+    """Device-wide reduction (mgpu::reduce) into a 1-element tensor; nothing
+    is written for an empty input."""
+    if not values.is_cuda or not values.is_contiguous():
+        raise TypeError("values must be a contiguous CUDA tensor")
+    code = _dtype_code(values, unsigned)
+    count = values.numel()
+    if out is None:
+        out = torch.zeros(1, dtype=values.dtype, device=values.device)
+    need = lib().mgpu_hip_reduce_workspace_bytes(count, code)
+    ws = _workspace(need, values.device)
+    _check(lib().mgpu_hip_reduce(
+        _ptr(values), count, ctypes.c_void_p(out.data_ptr()), code, OPS[op],
+        _ptr(ws), ws.numel(), _stream()))
     return out

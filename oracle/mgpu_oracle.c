@@ -19,8 +19,14 @@
  *   oracle_segreduce_* : closed form for the reference test's (index % 13)
  *       input with the reference test's generator and init=-1; numpy
  *       reduceat/fsum cross-checks; brute force.
+ *   oracle_lbs_segreduce_seg_plus_rank : closed form len * seg +
+ *       len * (len - 1) / 2 (mod 2^32) on the reference test's generator.
  *   oracle_interval_expand : numpy.repeat.
  *   oracle_spmv_* : scipy.sparse CSR product in float64.
+ *   oracle_scan_* : numpy cumsum / maximum.accumulate / minimum.accumulate and
+ *       the closed form of the reference's own scan test (50,000 times 1.01,
+ *       tests/test_scan.cu:13-16); the reduction against numpy sum/max/min and
+ *       the reference reduce test's all-ones input (tests/test_reduce.cu:14).
  */
 #include <stdint.h>
 #include <stddef.h>
@@ -236,6 +242,25 @@ ORACLE_API void oracle_segreduce_mod13(int count, const int* segments,
   }
 }
 
+/* lbs_segreduce, kernel_segreduce.hxx:303-404, with the functor the reference
+ * test defines for it, f(index, seg, rank) = seg + rank
+ * (tests/test_segreduce.cu:11-13), int32 '+': the load-balancing search hands
+ * every item its segment and its rank inside the segment, the values are
+ * reduced per segment, empty segments get init.                              */
+ORACLE_API void oracle_lbs_segreduce_seg_plus_rank(int count,
+  const int* segments, int num_segments, int* output, int init) {
+  for(int seg = 0; seg < num_segments; ++seg) {
+    int begin = segments[seg];
+    int end = (seg + 1 < num_segments) ? segments[seg + 1] : count;
+    int x = init;
+    for(int rank = 0; rank < end - begin; ++rank) {
+      int y = ADD_I32(seg, rank);
+      x = rank ? ADD_I32(x, y) : y;
+    }
+    output[seg] = x;
+  }
+}
+
 /* ------------------------------------------------------------------------- */
 /* spmv, kernel_segreduce.hxx:285-298: y[r] = sum_k matrix[k] * x[columns[k]]
  * over the row's nonzeros in order, plus_t, init 0 (empty row => 0); row
@@ -281,8 +306,11 @@ ORACLE_API void oracle_spmv_abs_f64(const void* matrix, const int* columns,
 /* Serial restatements of the CTA primitives' contracts, used to check the
  * wave64 device primitives.                                                  */
 
-/* cta_scan_t::scan, cta_scan.hxx:42-89: exclusive or inclusive scan of count
- * values with op; returns the reduction.                                     */
+/* cta_scan_t::scan, cta_scan.hxx:42-89, and the device-wide mgpu::scan,
+ * kernel_scan.hxx:11-165 (same contract with init = type_t()): exclusive or
+ * inclusive scan of count values with op; init is placed at out[0] of an
+ * exclusive scan and never folded; returns the reduction (init if count is
+ * 0).  mgpu::reduce, kernel_reduce.hxx:11-57, is that return value.          */
 #define DEF_SCAN(NAME, T, ADD)                                                \
 ORACLE_API T oracle_scan_##NAME(const T* in, int count, T* out, int op,       \
   T init, int inclusive) {                                                    \
@@ -297,6 +325,8 @@ ORACLE_API T oracle_scan_##NAME(const T* in, int count, T* out, int op,       \
   return x;                                                                   \
 }
 DEF_SCAN(i32, int32_t, ADD_I32)
+DEF_SCAN(u32, uint32_t, ADD_PLAIN)
 DEF_SCAN(i64, int64_t, ADD_I64)
+DEF_SCAN(u64, uint64_t, ADD_PLAIN)
 DEF_SCAN(f32, float, ADD_PLAIN)
 DEF_SCAN(f64, double, ADD_PLAIN)

@@ -159,6 +159,14 @@ def segreduce_mod13(count, segments, init=-1):
     return out
 
 
+def lbs_segreduce_seg_plus_rank(count, segments, init=-1):
+    s = _i32(segments)
+    out = np.empty(s.size, dtype=np.int32)
+    lib().oracle_lbs_segreduce_seg_plus_rank(int(count), _p(s), int(s.size), _p(out),
+                                             int(init))
+    return out
+
+
 def spmv(matrix, columns, vector, segments):
     m = np.ascontiguousarray(matrix)
     x = np.ascontiguousarray(vector, dtype=m.dtype)
@@ -183,9 +191,11 @@ def scan(values, op="plus", init=0, inclusive=False):
     v = np.ascontiguousarray(values)
     out = np.empty_like(v)
     name = {np.dtype(np.int32): "i32", np.dtype(np.int64): "i64",
+            np.dtype(np.uint32): "u32", np.dtype(np.uint64): "u64",
             np.dtype(np.float32): "f32", np.dtype(np.float64): "f64"}[v.dtype]
     fn = getattr(lib(), "oracle_scan_" + name)
-    ct = {"i32": ctypes.c_int32, "i64": ctypes.c_int64, "f32": ctypes.c_float,
+    ct = {"i32": ctypes.c_int32, "i64": ctypes.c_int64, "u32": ctypes.c_uint32,
+          "u64": ctypes.c_uint64, "f32": ctypes.c_float,
           "f64": ctypes.c_double}[name]
     fn.restype = ct
     fn.argtypes = [ctypes.c_void_p, ctypes.c_int, ctypes.c_void_p, ctypes.c_int,

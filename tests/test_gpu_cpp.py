@@ -33,3 +33,11 @@ def test_reference_style_load_balance(dev):
 
 def test_template_paths(dev):
     assert "all passed" in _run("test_templates")
+
+
+def test_reference_style_scan_and_reduce(dev):
+    assert "all passed" in _run("test_scan_reduce")
+
+
+def test_reference_style_lbs_segreduce(dev):
+    assert "all passed" in _run("test_lbs_segreduce", 4_000_000, 50_000)

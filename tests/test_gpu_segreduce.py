@@ -203,3 +203,22 @@ def test_full_size_config5_properties(dev, kind):
         nz = lens > 0
         assert torch.equal(got[nz], want[nz])
         assert torch.all(torch.isinf(got[~nz]) & (got[~nz] < 0))
+
+
+def test_lbs_segreduce_seg_plus_rank(oracle, dev):
+    """lbs_segreduce through the C ABI with the reference test's functor
+    (seg + rank, plus, init -1) on the layouts that stress tile boundaries."""
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    from util import segment_layouts
+    rng = np.random.default_rng(21)
+    nv = m.segreduce_tile_size(0)
+    for name, count, segs in segment_layouts(rng, nv):
+        got = m.lbs_segreduce_seg_plus_rank(count, _dev(segs), init=-1)
+        want = oracle.lbs_segreduce_seg_plus_rank(count, segs, init=-1)
+        assert np.array_equal(got.cpu().numpy(), want), name
+    for count, nseg, seed in ((10_000_000, 100, 0), (3_000_000, 100_000, 1), (40_000, 90_000, 2)):
+        segs = workloads.reference_test_segments(count, nseg, seed)
+        got = m.lbs_segreduce_seg_plus_rank(count, _dev(segs), init=-1)
+        want = oracle.lbs_segreduce_seg_plus_rank(count, segs, init=-1)
+        assert np.array_equal(got.cpu().numpy(), want), (count, nseg)

@@ -297,3 +297,73 @@ def test_scan_vs_numpy(oracle):
     assert out[0] == 9 and np.array_equal(out[1:], np.cumsum(v)[:-1])
     out, red = oracle.scan(v, "maximum", 0, inclusive=True)
     assert np.array_equal(out, np.maximum.accumulate(v))
+
+
+def test_scan_reference_test_vector(oracle):
+    """The reference's own scan test (tests/test_scan.cu:13-16): an exclusive
+    plus-scan of 50,000 copies of 1.01 in double; element i is the i-fold
+    running sum and the total is the 50,000-fold one.  Checked against the
+    exact product with the rounding bound of i additions."""
+    n = 50000
+    v = np.full(n, 1.01, dtype=np.float64)
+    out, red = oracle.scan(v, "plus", 0.0, inclusive=False)
+    i = np.arange(n, dtype=np.float64)
+    assert out[0] == 0.0
+    assert np.all(np.abs(out - 1.01 * i) <= (i + 1) * np.finfo(np.float64).eps * 1.01 * (i + 1))
+    assert abs(red - 1.01 * n) <= n * np.finfo(np.float64).eps * 1.01 * n
+    # the running sum is strictly increasing and each step adds 1.01 to rounding
+    assert np.all(np.abs(np.diff(out) - 1.01) <= 2 * np.spacing(out[1:]))
+
+
+def test_scan_all_types_and_ops_vs_numpy(oracle):
+    rng = np.random.default_rng(10)
+    for dt in (np.int32, np.uint32, np.int64, np.uint64):
+        v = rng.integers(0, 1 << 20, size=1234).astype(dt)
+        out, red = oracle.scan(v, "plus", 0, inclusive=True)
+        assert np.array_equal(out, np.cumsum(v, dtype=dt)) and red == v.sum(dtype=dt)
+        out, red = oracle.scan(v, "plus", 0, inclusive=False)
+        assert out[0] == 0 and np.array_equal(out[1:], np.cumsum(v, dtype=dt)[:-1])
+        out, red = oracle.scan(v, "minimum", 0, inclusive=True)
+        assert np.array_equal(out, np.minimum.accumulate(v)) and red == v.min()
+        # exclusive max: the placed zero is not folded into later elements
+        w = (v.astype(np.int64) - (1 << 21)).astype(np.int64) if dt == np.int64 else v
+        out, red = oracle.scan(w, "maximum", 0, inclusive=False)
+        assert out[0] == 0 and np.array_equal(out[1:], np.maximum.accumulate(w)[:-1])
+        assert red == w.max()
+    # wrap-around of integer sums
+    v = np.full(5, np.iinfo(np.int32).max, dtype=np.int32)
+    out, red = oracle.scan(v, "plus", 0, inclusive=True)
+    assert np.array_equal(out, np.cumsum(v.astype(np.int64)).astype(np.int32))
+    for dt in (np.float32, np.float64):
+        v = rng.standard_normal(999).astype(dt)
+        out, red = oracle.scan(v, "plus", 0, inclusive=True)
+        exact = np.cumsum(v.astype(np.longdouble))
+        bound = np.arange(1, v.size + 1) * np.finfo(dt).eps * np.cumsum(np.abs(v.astype(np.longdouble)))
+        assert np.all(np.abs(out - exact) <= bound)
+        out, red = oracle.scan(v, "maximum", 0, inclusive=True)
+        assert np.array_equal(out, np.maximum.accumulate(v)) and red == v.max()
+
+
+def test_reduce_reference_test_vector(oracle):
+    """The reference's reduce test folds an array of ones with plus
+    (tests/test_reduce.cu:14-20): the result is the count."""
+    for n in (1000, 1010, 123457):
+        out, red = oracle.scan(np.ones(n, dtype=np.int32), "plus", 0, inclusive=True)
+        assert red == n
+    out, red = oracle.scan(np.zeros(0, dtype=np.int32), "plus", 0, inclusive=False)
+    assert red == 0 and out.size == 0
+
+
+def test_lbs_segreduce_seg_plus_rank_closed_form(oracle):
+    """f = seg + rank summed over a segment of length L is L * seg +
+    L (L - 1) / 2 (mod 2^32); empty segments give init."""
+    from moderngpu_amd import workloads
+    for count, nseg, seed in ((100000, 1000, 0), (5000, 9000, 1), (1 << 20, 7, 2)):
+        segs = workloads.reference_test_segments(count, nseg, seed)
+        got = oracle.lbs_segreduce_seg_plus_rank(count, segs, init=-1)
+        ends = np.append(segs[1:], count).astype(np.int64)
+        L = ends - segs
+        want = (L * np.arange(nseg, dtype=np.int64) + L * (L - 1) // 2)
+        want = (want & 0xffffffff).astype(np.uint32).view(np.int32)
+        want = np.where(L == 0, np.int32(-1), want)
+        assert np.array_equal(got, want)
