@@ -16,6 +16,15 @@ using namespace mgpu;
 
 #define CHECK(cond, ...) do { if(!(cond)) { printf("FAILED %s:%d: ", __FILE__, __LINE__); printf(__VA_ARGS__); printf("\n"); return 1; } } while(0)
 
+// Keeps the left operand's tag and the right operand's count sum: associative,
+// not commutative.
+struct tagged_t { int tag; int sum; };
+struct keep_left_t {
+  MGPU_HOST_DEVICE tagged_t operator()(tagged_t a, tagged_t b) const {
+    return tagged_t { a.tag, a.sum + b.sum };
+  }
+};
+
 static int test_scan_constant(context_t& context) {
   typedef double type_t;
   int count = 50000;
@@ -33,15 +42,6 @@ static int test_scan_constant(context_t& context) {
   CHECK(std::fabs(total.data()[0] - want) <= 1e-12 * want, "total %.17g", total.data()[0]);
   return 0;
 }
-
-// Keeps the left operand's tag and the right operand's count sum: associative,
-// not commutative.
-struct tagged_t { int tag; int sum; };
-struct keep_left_t {
-  MGPU_HOST_DEVICE tagged_t operator()(tagged_t a, tagged_t b) const {
-    return tagged_t { a.tag, a.sum + b.sum };
-  }
-};
 
 static int test_scan_sizes(context_t& context) {
   for(int count : { 1, 100, 16384, 16385, 70001, 3000017 }) {
@@ -96,6 +96,21 @@ static int test_scan_two_levels(context_t& context) {
     x += (i & 3) + 1;
   }
   CHECK(from_mem(total)[0] == x, "two-level total");
+
+  // The same with a value type that takes the three-launch path, enough
+  // tiles that the partials need a second level.
+  int count2 = 256 * 16500 + 77;
+  std::vector<tagged_t> host(count2);
+  for(int i = 0; i < count2; ++i) host[i] = tagged_t { i, 1 };
+  mem_t<tagged_t> in = to_mem(host, context);
+  mem_t<tagged_t> out(count2, context), red(1, context);
+  scan<scan_type_inc, launch_t>(in.data(), count2, out.data(), keep_left_t(),
+    red.data(), context);
+  std::vector<tagged_t> z = from_mem(out);
+  for(int i = 0; i < count2; ++i)
+    CHECK(z[i].tag == 0 && z[i].sum == i + 1, "two-level tagged scan[%d] = (%d, %d)", i, z[i].tag, z[i].sum);
+  tagged_t r = from_mem(red)[0];
+  CHECK(r.tag == 0 && r.sum == count2, "two-level tagged total (%d, %d)", r.tag, r.sum);
   return 0;
 }
 
