@@ -176,8 +176,7 @@ struct lbs_partition_scatter_f {
     // Boundaries b with m_j < spacing * b <= m_{j+1} have exactly j + 1
     // starts in front of them.  The clamps keep malformed (unsorted) input
     // from writing outside p.  Only the first of them can be closer than
-    // `snap` items to the start of segment j; all threads of a wavefront
-    // stay together here so that they can resolve those cases jointly.
+    // `snap` items to the start of segment j.
     int lane = tid % warp_size;
     // tile_at[e] = tile holding merged position m_{j0 + e}.
     int tile_at[vt + 1];
@@ -185,42 +184,45 @@ struct lbs_partition_scatter_f {
     for(int e = 0; e <= vt; ++e)
       tile_at[e] = tile_of(min(max(starts[e] + j0 + e, 0), total));
 
+    // Few segments have a split behind them (one in spacing / mean segment
+    // length), so everything but the test for it sits inside the branch.
     PRAGMA_UNROLL
     for(int e = 0; e < vt; ++e) {
       int j = j0 + e;
-      int first = 0, n = 0;
-      if(j < num_segments) {
-        first = tile_at[e] + 1;
-        n = max(tile_at[e + 1] - first + 1, 0);
-      }
+      int first = tile_at[e] + 1;
+      int n = (j < num_segments) ? tile_at[e + 1] - tile_at[e] : 0;
 
-      if constexpr(snap > 0) {
-        // First split: the snapped item index may lie in front of the start
-        // of segment j and of starts before it.  The wavefront counts them
-        // for one such split at a time: lane l looks at start j - l.
-        int a = first * spacing - (j + 1);
-        int a_snap = a - a % snap;
-        bool inner = n > 0 && first * spacing < total;
-        bool look = inner && starts[e] > a_snap;
-        int back = 0;
-        lanemask_t pending = ballot(look);
-        while(pending) {
-          int src = (int)__builtin_ctzll(pending);
-          pending &= pending - 1;
-          int src_j = readlane(j, src);
-          int src_snap = readlane(a_snap, src);
-          int idx = src_j - lane;
-          bool later = lane < window && idx >= 0 &&
-            (int)segments[idx] > src_snap;
-          int c = __builtin_popcountll(ballot(later));
-          if(lane == src) back = c;
-        }
-        if(n > 0) {
+      if(n > 0) {
+        if constexpr(snap > 0) {
+          // First split: the snapped item index may lie in front of the
+          // start of segment j and of starts before it.  The thread counts
+          // them, eight starts a step, all of a step's loads in flight
+          // together; one step is enough for most splits.
+          int a = first * spacing - (j + 1);
+          int a_snap = a - a % snap;
+          bool inner = first * spacing < total;
+          int back = 0;
+          if(inner && starts[e] > a_snap) {
+            back = 1;
+            bool more = true;
+            while(more && back < window && j - back >= 0) {
+              int top = j - back;             // nearest start not yet seen
+              int v[8];
+              PRAGMA_UNROLL
+              for(int q = 0; q < 8; ++q)
+                v[q] = segments[max(top - q, 0)];
+              PRAGMA_UNROLL
+              for(int q = 0; q < 8; ++q) {
+                if(more && top - q >= 0 && v[q] > a_snap) ++back;
+                else more = false;
+              }
+            }
+          }
           if(inner && back < window) write_pair(first, a_snap, j + 1 - back);
           else write_pair(first, a, j + 1);
-        }
-      } else if(n > 0)
-        write_inside(first, j + 1);
+        } else
+          write_inside(first, j + 1);
+      }
 
       // The other splits inside segment j: written by the thread itself when
       // there are few, by the whole wavefront when the segment spans many
