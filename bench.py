@@ -302,11 +302,11 @@ FACTORIES = {
 # FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by what the same counters
 # read for a plain copy of known size.  None until measured.
 TRAFFIC_BYTES = {
-    # profiles/segreduce_tile_f__c2_segreduce_f32.md: FETCH 133,562.5 KiB x 2.000
-    # + WRITE 4,279.3 KiB x 1.000
-    "c2_segreduce_f32": int((133562.5 * 2.000 + 4279.3) * 1024),
+    # profiles/segreduce_tile_f__c2_segreduce_f32.md: FETCH 133,785.8 KiB x 2.000
+    # + WRITE 4,286.2 KiB x 1.000
+    "c2_segreduce_f32": int((133785.8 * 2.000 + 4286.2) * 1024),
     # profiles/transform_lbs_f__c3_load_balance_search.md
-    "c3_load_balance_search": int((33634.5 * 2.000 + 1048977.7) * 1024),
+    "c3_load_balance_search": int((33529.9 * 2.000 + 1048576.1) * 1024),
 }
 
 
