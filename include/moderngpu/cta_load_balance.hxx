@@ -226,12 +226,78 @@ MGPU_DEVICE inline void store_consecutive(type_t* dest,
 
 ////////////////////////////////////////////////////////////////////////////////
 
-// Kept for source compatibility: where a thread's slice of the merge starts.
+// Where a thread's slice of the tile's merge begins (interface after
+// src/moderngpu/cta_load_balance.hxx:9-65).  `range` is the range of the
+// starts that were loaded: the tile's own, one more in front when there is
+// one (the segment that is open when the tile begins) and one more behind
+// when items remain past the tile.
 struct lbs_placement_t {
-  merge_range_t range;    // range of loaded values
-  int a_index;            // first item of the thread
-  int b_index;            // segment of that item
+  merge_range_t range;
+  int a_index;            // first item the thread merges
+  int b_index;            // segment that item belongs to
 };
+
+// Loads the tile's segment starts into b_shared (behind them, up to slot
+// nv + 1, `count` as a sentinel) and finds by a merge-path search in LDS
+// where thread tid's slice of vt merged elements begins.  b_shared must hold
+// nt * vt + 2 - range.a_count() ints.  Two barriers.
+template<int nt, int vt, typename segments_it>
+MGPU_DEVICE lbs_placement_t cta_load_balance_place(int tid,
+  merge_range_t range, int count, segments_it segments, int num_segments,
+  int* b_shared) {
+
+  int preceding = range.b_begin > 0;
+  range.b_begin -= preceding;
+  if(range.b_end < num_segments && range.a_end < count) ++range.b_end;
+
+  int loaded = range.b_count();
+  int sentinels = nt * vt + 1 + preceding - loaded - range.a_count();
+  for(int i = tid; i < loaded; i += nt)
+    b_shared[i] = segments[range.b_begin + i];
+  for(int i = tid; i < sentinels; i += nt)
+    b_shared[loaded + i] = count;
+  __syncthreads();
+
+  // The preceding start has been consumed before the tile begins: skip it.
+  int diag = vt * tid + preceding;
+  int mp = merge_path<bounds_upper>(counting_iterator_t<int>(range.a_begin),
+    range.a_count(), b_shared, loaded + sentinels, diag, less_t<int>());
+  __syncthreads();
+
+  // diag - mp starts lie in front of the slice; the last of them is the
+  // segment of the slice's first item.
+  return lbs_placement_t { range, range.a_begin + mp,
+    range.b_begin + (diag - mp) - 1 };
+}
+
+// What cta_load_balance_fill leaves behind: shared[i] = segment of tile item
+// i for i in [0, range.a_count()), and the start of segment s at
+// shared[b_offset + s] (interface after cta_load_balance.hxx:67-105).
+struct lbs_fill_t {
+  merge_range_t range;
+  int b_offset;
+};
+
+template<int nt, int vt, typename segments_it, typename partition_it>
+MGPU_DEVICE lbs_fill_t cta_load_balance_fill(int count, segments_it segments,
+  int num_segments, int tid, int cta, partition_it partitions, int* shared) {
+
+  merge_range_t range = detail::tile_range(count, num_segments, cta, nt * vt,
+    partitions[cta], partitions[cta + 1]);
+  int* a_shared = shared - range.a_begin;
+  int* b_shared = shared + range.a_count();
+  lbs_placement_t placement = cta_load_balance_place<nt, vt>(tid, range,
+    count, segments, num_segments, b_shared);
+  b_shared -= placement.range.b_begin;
+
+  int item = placement.a_index, segment = placement.b_index;
+  iterate<vt>([&](int) {
+    if(item < b_shared[segment + 1]) a_shared[item++] = segment;
+    else ++segment;
+  });
+  __syncthreads();
+  return lbs_fill_t { range, range.a_count() - placement.range.b_begin };
+}
 
 template<int nt, int vt>
 struct cta_load_balance_t {
@@ -254,7 +320,7 @@ struct cta_load_balance_t {
   struct result_t {
     lbs_placement_t placement;
     merge_range_t merge_range;
-    int merge_flags;                // not produced by this implementation
+    int merge_flags;                // thread order: bit i of the serial merge
 
     // Strided order: element i is tile item nt * i + tid.
     array_t<int, vt> indices;       // global item index
@@ -350,31 +416,48 @@ struct cta_load_balance_t {
     __syncthreads();
   }
 
-  // Full search: (index, segment, rank) per item in strided order.  Items
-  // past the end of the tile get segment b_begin and rank -1.
+  // The CTA-level search with everything the reference's returns
+  // (cta_load_balance.hxx:107-184): the thread's placement, the bits of its
+  // serial merge (bit i set: step i of the vt + 1 steps took an item, clear:
+  // it moved on to the next segment), and per item in strided order the global
+  // index, its segment and its rank; items past the end of the tile get
+  // segment b_begin and rank -1.  This is the thread-per-diagonal form --
+  // a merge-path search and vt + 1 dependent LDS reads per thread -- for
+  // callers that need placement or merge bits; the library's own kernels
+  // decode tiles with fill() above, which has neither.
   template<typename segments_it, typename partition_it>
   MGPU_DEVICE result_t load_balance(int count, segments_it segments,
     int num_segments, int tid, int cta, partition_it partitions,
     storage_t& storage) const {
 
-    merge_range_t range = fill(count, segments, num_segments, tid, cta,
-      partitions, storage);
-    int a_count = range.a_count();
-    const int* slots = storage.indices;
-    const int* starts = storage.indices + starts_offset(a_count);
+    merge_range_t range = detail::tile_range(count, num_segments, cta, nv,
+      partitions[cta], partitions[cta + 1]);
+    int* a_shared = storage.indices - range.a_begin;
+    int* b_shared = storage.indices + range.a_count();
+    lbs_placement_t placement = cta_load_balance_place<nt, vt>(tid, range,
+      count, segments, num_segments, b_shared);
+    b_shared -= placement.range.b_begin;
+
+    int item = placement.a_index, segment = placement.b_index;
+    int merge_flags = 0;
+    iterate<vt + 1>([&](int i) {
+      bool take = item < b_shared[segment + 1];
+      if(take && i < vt) a_shared[item++] = segment;
+      else ++segment;
+      merge_flags |= (int)take << i;
+    });
+    __syncthreads();
 
     result_t result;
+    result.placement = placement;
     result.merge_range = range;
-    result.placement = lbs_placement_t { range, range.a_begin,
-      range.b_begin - 1 };
-    result.merge_flags = 0;
+    result.merge_flags = merge_flags;
     iterate<vt>([&](int i) {
       int j = nt * i + tid;
       result.indices[i] = range.a_begin + j;
-      if(j < a_count) {
-        int rel = slots[layout_t::index(j)];
-        result.segments[i] = range.b_begin - 1 + rel;
-        result.ranks[i] = result.indices[i] - starts[rel];
+      if(j < range.a_count()) {
+        result.segments[i] = storage.indices[j];
+        result.ranks[i] = result.indices[i] - b_shared[result.segments[i]];
       } else {
         result.segments[i] = range.b_begin;
         result.ranks[i] = -1;

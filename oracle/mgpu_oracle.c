@@ -21,6 +21,10 @@
  *       reduceat/fsum cross-checks; brute force.
  *   oracle_lbs_segreduce_seg_plus_rank : closed form len * seg +
  *       len * (len - 1) / 2 (mod 2^32) on the reference test's generator.
+ *   oracle_cta_load_balance : per-item (segment, rank) against
+ *       oracle_transform_lbs on the tile's items; every tile item written by
+ *       exactly one thread; popcount of a thread's low vt merge bits = items it
+ *       takes; placements consecutive (a thread ends where the next begins).
  *   oracle_interval_expand : numpy.repeat.
  *   oracle_spmv_* : scipy.sparse CSR product in float64.
  *   oracle_scan_* : numpy cumsum / maximum.accumulate / minimum.accumulate and
@@ -300,6 +304,76 @@ ORACLE_API void oracle_spmv_abs_f64(const void* matrix, const int* columns,
     }
     output[row] = x;
   }
+}
+
+/* ------------------------------------------------------------------------- */
+/* cta_load_balance_place and cta_load_balance_t::load_balance,
+ * cta_load_balance.hxx:16-65 and :107-184, for tile `cta` of nv = nt * vt merged
+ * elements, thread by thread.  Per thread tid: a_index[tid], b_index[tid]
+ * (placement) and merge_flags[tid]; per thread and i < vt, at [tid * vt + i]:
+ * the global index, segment and rank of tile item nt * i + tid (segment
+ * b_begin and rank -1 past the end of the tile).  range_out = the loaded
+ * range {a_begin, a_end, b_begin, b_end} of the placement.                   */
+ORACLE_API void oracle_cta_load_balance(int count, const int* segments,
+  int num_segments, int nt, int vt, int cta, int* a_index, int* b_index,
+  int* merge_flags, int* indices, int* segs, int* ranks, int range_out[4]) {
+  int nv = nt * vt;
+  int total = count + num_segments;
+  int diag0 = nv * cta, diag1 = diag0 + nv < total ? diag0 + nv : total;
+  int mp0 = oracle_merge_path(NULL, count, segments, num_segments, diag0, 1);
+  int mp1 = oracle_merge_path(NULL, count, segments, num_segments, diag1, 1);
+  int a_begin = mp0, a_end = mp1, b_begin = diag0 - mp0, b_end = diag1 - mp1;
+  int a_count = a_end - a_begin;
+
+  /* cta_load_balance.hxx:21-44: starts as loaded, then `count` sentinels.    */
+  int preceding = b_begin > 0;
+  int lb = b_begin - preceding, le = b_end;
+  if(le < num_segments && a_end < count) ++le;
+  int loaded = le - lb;
+  int sentinels = nv + 1 + preceding - loaded - a_count;
+  int n = loaded + sentinels;
+  int* b = (int*)__builtin_alloca(sizeof(int) * (size_t)(n + 2));
+  for(int i = 0; i < loaded; ++i) b[i] = segments[lb + i];
+  for(int i = 0; i < sentinels; ++i) b[loaded + i] = count;
+  int* seg_of = (int*)__builtin_alloca(sizeof(int) * (size_t)(nv + vt + 2));
+
+  range_out[0] = a_begin; range_out[1] = a_end;
+  range_out[2] = lb; range_out[3] = le;
+
+  for(int tid = 0; tid < nt; ++tid) {
+    /* :49-63: merge path of (a_begin + i) against b with bounds_upper.       */
+    int diag = vt * tid + preceding;
+    int lo = diag - n > 0 ? diag - n : 0;
+    int hi = diag < a_count ? diag : a_count;
+    while(lo < hi) {
+      int mid = (lo + hi) / 2;
+      int a_key = a_begin + mid, b_key = b[diag - 1 - mid];
+      if(a_key < b_key) lo = mid + 1; else hi = mid;
+    }
+    int mp = lo;
+    a_index[tid] = a_begin + mp;
+    b_index[tid] = lb + (diag - mp) - 1;
+
+    /* :129-143: vt + 1 merge steps.                                          */
+    int item = a_index[tid], segment = b_index[tid], flags = 0;
+    for(int i = 0; i <= vt; ++i) {
+      int p = item < b[segment + 1 - lb];
+      if(p && i < vt) { seg_of[item - a_begin] = segment; ++item; }
+      else ++segment;
+      flags |= p << i;
+    }
+    merge_flags[tid] = flags;
+  }
+  /* :149-160: strided read-back.                                             */
+  for(int tid = 0; tid < nt; ++tid)
+    for(int i = 0; i < vt; ++i) {
+      int j = nt * i + tid, at = tid * vt + i;
+      indices[at] = a_begin + j;
+      if(j < a_count) {
+        segs[at] = seg_of[j];
+        ranks[at] = indices[at] - b[segs[at] - lb];
+      } else { segs[at] = b_begin; ranks[at] = -1; }
+    }
 }
 
 /* ------------------------------------------------------------------------- */

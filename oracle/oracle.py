@@ -167,6 +167,24 @@ def lbs_segreduce_seg_plus_rank(count, segments, init=-1):
     return out
 
 
+def cta_load_balance(count, segments, nt, vt, cta):
+    """One tile of cta_load_balance_t::load_balance, thread by thread."""
+    s = _i32(segments)
+    a_index = np.empty(nt, dtype=np.int32)
+    b_index = np.empty(nt, dtype=np.int32)
+    flags = np.empty(nt, dtype=np.int32)
+    indices = np.empty(nt * vt, dtype=np.int32)
+    segs = np.empty(nt * vt, dtype=np.int32)
+    ranks = np.empty(nt * vt, dtype=np.int32)
+    rng = np.empty(4, dtype=np.int32)
+    lib().oracle_cta_load_balance(int(count), _p(s), int(s.size), int(nt), int(vt),
+                                  int(cta), _p(a_index), _p(b_index), _p(flags),
+                                  _p(indices), _p(segs), _p(ranks), _p(rng))
+    return {"a_index": a_index, "b_index": b_index, "merge_flags": flags,
+            "indices": indices.reshape(nt, vt), "segments": segs.reshape(nt, vt),
+            "ranks": ranks.reshape(nt, vt), "range": rng}
+
+
 def spmv(matrix, columns, vector, segments):
     m = np.ascontiguousarray(matrix)
     x = np.ascontiguousarray(vector, dtype=m.dtype)

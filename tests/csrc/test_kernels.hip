@@ -5,6 +5,8 @@
 #include <moderngpu/cta_reduce.hxx>
 #include <moderngpu/cta_scan.hxx>
 #include <moderngpu/cta_segscan.hxx>
+#include <moderngpu/cta_load_balance.hxx>
+#include <moderngpu/search.hxx>
 #include <moderngpu/transform.hxx>
 
 using namespace mgpu;
@@ -135,6 +137,56 @@ void run_shfl(const int* in, int* out, int mode, int offset, int width) {
   }, 1, context);
 }
 
+// One CTA per tile runs cta_load_balance_t::load_balance (splits from
+// load_balance_partitions with spacing nv) and dumps everything it returns;
+// with fill_mode, cta_load_balance_fill instead: the segment of every tile item
+// and (through b_offset) the rank.
+template<int nt, int vt>
+void run_load_balance(int count, const int* segments, int num_segments,
+  int* partitions, int* a_index, int* b_index, int* merge_flags, int* indices,
+  int* segs, int* ranks, int* ranges, int fill_mode) {
+  bare_context_t context;
+  enum { nv = nt * vt };
+  int num_tiles = div_up(count + num_segments, (int)nv);
+  load_balance_partitions_into((int64_t)count, segments, num_segments, nv,
+    partitions, context);
+  cta_launch<nt>([=]MGPU_DEVICE(int tid, int cta) {
+    typedef cta_load_balance_t<nt, vt> lbs_t;
+    __shared__ typename lbs_t::storage_t storage;
+    size_t thread = (size_t)cta * nt + tid;
+    if(fill_mode) {
+      lbs_fill_t fill = cta_load_balance_fill<nt, vt>(count, segments,
+        num_segments, tid, cta, partitions, storage.indices);
+      for(int i = 0; i < vt; ++i) {
+        int j = nt * i + tid;
+        size_t at = thread * vt + i;
+        indices[at] = fill.range.a_begin + j;
+        if(j < fill.range.a_count()) {
+          segs[at] = storage.indices[j];
+          ranks[at] = indices[at] - storage.indices[fill.b_offset + segs[at]];
+        } else { segs[at] = fill.range.b_begin; ranks[at] = -1; }
+      }
+      return;
+    }
+    typename lbs_t::result_t r = lbs_t().load_balance(count, segments,
+      num_segments, tid, cta, partitions, storage);
+    a_index[thread] = r.placement.a_index;
+    b_index[thread] = r.placement.b_index;
+    merge_flags[thread] = r.merge_flags;
+    for(int i = 0; i < vt; ++i) {
+      indices[thread * vt + i] = r.indices[i];
+      segs[thread * vt + i] = r.segments[i];
+      ranks[thread * vt + i] = r.ranks[i];
+    }
+    if(!tid) {
+      ranges[4 * cta + 0] = r.placement.range.a_begin;
+      ranges[4 * cta + 1] = r.placement.range.a_end;
+      ranges[4 * cta + 2] = r.placement.range.b_begin;
+      ranges[4 * cta + 3] = r.placement.range.b_end;
+    }
+  }, num_tiles, context);
+}
+
 #define BY_NT(fn, ...)                                                        \
   switch(nt) {                                                                \
     case 64: fn<64>(__VA_ARGS__); break;                                      \
@@ -221,4 +273,16 @@ API int tk_scan_bool(int nt, const int* in, int* out, int* red) {
 API int tk_shfl(const int* in, int* out, int mode, int offset, int width) {
   run_shfl(in, out, mode, offset, width);
   return finish();
+}
+
+API int tk_load_balance(int nt, int vt, int count, const int* segments,
+  int num_segments, int* partitions, int* a_index, int* b_index,
+  int* merge_flags, int* indices, int* segs, int* ranks, int* ranges,
+  int fill_mode) {
+#define LB(NT, VT) if(NT == nt && VT == vt) { run_load_balance<NT, VT>(count,  \
+  segments, num_segments, partitions, a_index, b_index, merge_flags, indices, \
+  segs, ranks, ranges, fill_mode); return finish(); }
+  LB(64, 3) LB(128, 7) LB(128, 11) LB(256, 4) LB(256, 16) LB(512, 12)
+#undef LB
+  return -1;
 }

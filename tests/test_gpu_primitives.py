@@ -242,3 +242,43 @@ def test_shuffles_and_lane_queries(tk, dev):
     assert (run(4) == int(x[0])).all()      # all-reduce with left projection
     assert np.array_equal(run(5), lane)
     assert (run(6) == int((x & 1).sum())).all()
+
+
+@pytest.mark.parametrize("nt,vt", [(64, 3), (128, 7), (128, 11), (256, 4), (256, 16), (512, 12)])
+def test_cta_load_balance_placement_and_merge_flags(tk, dev, oracle, nt, vt):
+    """cta_load_balance_t::load_balance (placement, merge bits, strided
+    index/segment/rank) and cta_load_balance_fill against the thread-by-thread
+    CPU restatement, tile by tile."""
+    import torch
+    rng = np.random.default_rng(nt * 100 + vt)
+    nv = nt * vt
+    cases = [(5 * nv + 17, 40), (3 * nv, 2 * nv + 5), (nv // 2, 7), (4 * nv + 1, 900)]
+    for count, nseg in cases:
+        segs = np.zeros(nseg, dtype=np.int32)
+        segs[1:] = np.sort(rng.integers(0, count + 1, size=nseg - 1))
+        tiles = (count + nseg + nv - 1) // nv
+        d_segs = _dev(torch, segs)
+        parts = torch.zeros(tiles + 1, dtype=torch.int32, device="cuda")
+        outs = {k: torch.full((tiles * nt,), -7, dtype=torch.int32, device="cuda")
+                for k in ("a_index", "b_index", "merge_flags")}
+        big = {k: torch.full((tiles * nt * vt,), -7, dtype=torch.int32, device="cuda")
+               for k in ("indices", "segments", "ranks")}
+        ranges = torch.zeros(4 * tiles, dtype=torch.int32, device="cuda")
+        for fill_mode in (0, 1):
+            rc = tk.tk_load_balance(nt, vt, count, _p(d_segs), nseg, _p(parts),
+                                    _p(outs["a_index"]), _p(outs["b_index"]),
+                                    _p(outs["merge_flags"]), _p(big["indices"]),
+                                    _p(big["segments"]), _p(big["ranks"]), _p(ranges),
+                                    fill_mode)
+            assert rc == 0
+            got = {k: v.cpu().numpy().reshape(tiles, nt) for k, v in outs.items()}
+            gbig = {k: v.cpu().numpy().reshape(tiles, nt, vt) for k, v in big.items()}
+            grange = ranges.cpu().numpy().reshape(tiles, 4)
+            for cta in range(tiles):
+                want = oracle.cta_load_balance(count, segs, nt, vt, cta)
+                for k in ("indices", "segments", "ranks"):
+                    assert np.array_equal(gbig[k][cta], want[k]), (count, nseg, cta, k, fill_mode)
+                if not fill_mode:
+                    for k in ("a_index", "b_index", "merge_flags"):
+                        assert np.array_equal(got[k][cta], want[k]), (count, nseg, cta, k)
+                    assert np.array_equal(grange[cta], want["range"]), (count, nseg, cta)

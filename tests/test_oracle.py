@@ -367,3 +367,58 @@ def test_lbs_segreduce_seg_plus_rank_closed_form(oracle):
         want = (want & 0xffffffff).astype(np.uint32).view(np.int32)
         want = np.where(L == 0, np.int32(-1), want)
         assert np.array_equal(got, want)
+
+
+def test_cta_load_balance_structure(oracle):
+    """The thread-by-thread tile search: per-item results agree with the
+    device-wide search (pinned above), every item of the tile is produced by
+    exactly one thread, a thread's merge bits count the items it takes, and
+    consecutive threads' placements chain (thread t + 1 begins where the vt
+    merge steps of thread t end)."""
+    rng = np.random.default_rng(17)
+    for nt, vt, count, nseg in ((64, 3, 1000, 300), (128, 7, 5000, 40), (64, 3, 700, 2000),
+                                (128, 11, 20000, 3000)):
+        segs = np.zeros(nseg, dtype=np.int32)
+        segs[1:] = np.sort(rng.integers(0, count + 1, size=nseg - 1))
+        want_seg, want_rank = oracle.transform_lbs(count, segs)
+        nv = nt * vt
+        tiles = (count + nseg + nv - 1) // nv
+        seen = np.zeros(count, dtype=np.int32)
+        for cta in range(tiles):
+            r = oracle.cta_load_balance(count, segs, nt, vt, cta)
+            idx, sg, rk = r["indices"], r["segments"], r["ranks"]
+            valid = rk >= 0
+            a_begin, a_end = int(r["range"][0]), int(r["range"][1])
+            assert np.all((idx[valid] >= a_begin) & (idx[valid] < a_end))
+            assert np.array_equal(sg[valid], want_seg[idx[valid]])
+            assert np.array_equal(rk[valid], want_rank[idx[valid]])
+            seen[idx[valid]] += 1
+            flags = r["merge_flags"].astype(np.int64)
+            taken = np.array([bin(int(f) & ((1 << vt) - 1)).count("1") for f in flags])
+            # chaining: next thread's a_index = this thread's a_index + items taken
+            assert np.array_equal(r["a_index"][1:], (r["a_index"] + taken)[:-1])
+            # and its b_index advances by the starts passed (vt - items taken)
+            assert np.array_equal(r["b_index"][1:], (r["b_index"] + vt - taken)[:-1])
+            # the first thread starts at the tile's first item, in the open segment
+            assert r["a_index"][0] == a_begin
+            if a_begin < a_end:
+                assert r["b_index"][0] + (1 if (flags[0] & 1) == 0 else 0) <= want_seg[a_begin]
+        assert np.all(seen == 1)
+
+
+def test_cta_load_balance_hand_example(oracle):
+    """segments = {0, 3, 3, 7}, 10 items, tiles of 4 threads x 2: worked by
+    hand from the merge order  s0 0 1 2 s1 s2 3 4 | 5 6 s3 7 8 9."""
+    segs = np.array([0, 3, 3, 7], dtype=np.int32)
+    # oracle_cta_load_balance needs nt, vt only as numbers: 4 x 2.
+    r = oracle.cta_load_balance(10, segs, 4, 2, 0)
+    # tile 0 = merged positions [0, 8): starts s0,s1,s2 and items 0..4
+    assert list(r["range"][:2]) == [0, 5]
+    assert list(r["a_index"]) == [0, 1, 3, 3]
+    assert list(r["b_index"]) == [-1, 0, 0, 2]
+    # thread 0: s0 (bit 0 clear), item 0 (bit 1 set), then peeks item 1 (bit 2 set)
+    assert [int(f) & 3 for f in r["merge_flags"]] == [0b10, 0b11, 0b00, 0b11]
+    r = oracle.cta_load_balance(10, segs, 4, 2, 1)
+    assert list(r["range"][:2]) == [5, 10]
+    assert list(r["a_index"]) == [5, 7, 8, 10]
+    assert list(r["b_index"]) == [2, 2, 3, 3]
