@@ -77,6 +77,12 @@ def make_c2(copies):
         from oracle import oracle
         return lambda: oracle.segreduce(w["values"], w["segments"], "plus", 0.0)
     wk.cpu = cpu
+
+    def cpu_threads(threads):
+        from oracle import oracle
+        return lambda: oracle.segreduce_threads(w["values"], w["segments"], "plus", 0.0,
+                                                threads=threads)
+    wk.cpu_threads = cpu_threads
     return wk
 
 
@@ -212,6 +218,12 @@ def make_c5(copies, kind):
         from oracle import oracle
         return lambda: oracle.segreduce(w["values"], w["segments"], w["op"], w["init"])
     wk.cpu = cpu
+
+    def cpu_threads(threads):
+        from oracle import oracle
+        return lambda: oracle.segreduce_threads(w["values"], w["segments"], w["op"],
+                                                w["init"], threads=threads)
+    wk.cpu_threads = cpu_threads
     return wk
 
 
@@ -341,19 +353,37 @@ def time_kernel_events(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps / 1e3
 
 
-def cpu_baseline(wk, budget_s=4.0):
-    run = wk.cpu()
+def _time_cpu(run, budget_s):
     reps, t_total = 0, 0.0
     while reps < 1 or (t_total < budget_s and reps < 50):
         t0 = time.perf_counter()
         run()
         t_total += time.perf_counter() - t0
         reps += 1
-    sec = t_total / reps
-    return {"value": wk.bytes / sec / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
-            "items_per_s": wk.items / sec,
-            "sample": "full workload, %d repetition(s), single thread, gcc -O3 -march=native "
-                      "(host has %d logical cores)" % (reps, os.cpu_count() or 0)}
+    return t_total / reps, reps
+
+
+def cpu_baseline(wk, budget_s=4.0):
+    """The CPU checker's loop timed on this host: single thread (what the
+    reference's own tests run) and, where the workload splits by segment
+    ranges, all the cores this process may use."""
+    sec1, reps1 = _time_cpu(wk.cpu(), budget_s)
+    res = {"value": wk.bytes / sec1 / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+           "items_per_s": wk.items / sec1,
+           "sample": "full workload, %d repetition(s), single thread, gcc -O3 -march=native "
+                     "(host reports %d logical cores)" % (reps1, os.cpu_count() or 0)}
+    make = getattr(wk, "cpu_threads", None)
+    cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores) or cores))
+    if make is not None and cores > 1:
+        secn, repsn = _time_cpu(make(cores), budget_s)
+        res = {"value": wk.bytes / secn / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
+               "items_per_s": wk.items / secn,
+               "single_thread_value": wk.bytes / sec1 / 1e9,
+               "sample": "full workload, %d repetition(s) on %d threads over contiguous "
+                         "segment ranges (and %d single-threaded: the single_thread_value), "
+                         "gcc -O3 -march=native" % (repsn, cores, reps1)}
+    return res
 
 
 def main():
@@ -418,6 +448,15 @@ def main():
         torch.cuda.empty_cache()
         return res
 
+    props = torch.cuda.get_device_properties(0)
+    device = {"name": props.name, "compute_units": props.multi_processor_count,
+              "hbm_peak_used_GBps": HBM_PEAK_GBPS}
+    # memory clock x bus width, double data rate, as the runtime reports them
+    clock_khz = getattr(props, "memory_clock_rate", 0)
+    bus_bits = getattr(props, "memory_bus_width", 0)
+    if clock_khz and bus_bits:
+        device["hbm_peak_from_device_properties_GBps"] = 2.0 * clock_khz * 1e3 * bus_bits / 8 / 1e9
+
     main_res = measure(args.workload, not args.no_cpu)
     others = {}
     for key in [k for k in args.extra.split(",") if k and k != args.workload]:
@@ -439,6 +478,7 @@ def main():
     }
     if "cpu_baseline" in main_res:
         line["cpu_baseline"] = main_res["cpu_baseline"]
+    line["device"] = device
     if others:
         line["others"] = others
     print(json.dumps(line))

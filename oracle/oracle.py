@@ -152,6 +152,37 @@ def segreduce(values, segments, op="plus", init=0):
     return out
 
 
+def segreduce_threads(values, segments, op="plus", init=0, threads=1):
+    """The same loop run by `threads` host threads, each over a contiguous
+    range of segments holding about the same number of items (the C call
+    releases the GIL).  Used as the all-cores CPU baseline."""
+    from concurrent.futures import ThreadPoolExecutor
+    v = np.ascontiguousarray(values)
+    s = _i32(segments)
+    out = np.empty(s.size, dtype=v.dtype)
+    ini = np.array([init], dtype=v.dtype)
+    if threads <= 1 or s.size < 2 * threads:
+        return segreduce(values, segments, op, init)
+    # segment index where each thread starts: balanced by items
+    cuts = np.searchsorted(s, np.arange(1, threads) * (v.size // threads), side="left")
+    bounds = [0] + [int(c) for c in cuts] + [int(s.size)]
+    fn = lib().oracle_segreduce
+    dt, opc = DTYPES[v.dtype], OPS[op]
+    sp, op_, vp, ip = s.ctypes.data, out.ctypes.data, _p(v), _p(ini)
+
+    def run(k):
+        b, e = bounds[k], bounds[k + 1]
+        if e <= b:
+            return 0
+        end_item = int(s[e]) if e < s.size else int(v.size)
+        return fn(vp, end_item, ctypes.c_void_p(sp + 4 * b), e - b,
+                  ctypes.c_void_p(op_ + v.itemsize * b), dt, opc, ip)
+
+    with ThreadPoolExecutor(max_workers=threads) as pool:
+        assert all(rc == 0 for rc in pool.map(run, range(threads)))
+    return out
+
+
 def segreduce_mod13(count, segments, init=-1):
     s = _i32(segments)
     out = np.empty(s.size, dtype=np.int32)
