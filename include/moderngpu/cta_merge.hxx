@@ -49,8 +49,8 @@ MGPU_HOST_DEVICE int merge_path(keys_it keys, merge_range_t range,
 template<bounds_t bounds, bool range_check, typename type_t, typename comp_t>
 MGPU_HOST_DEVICE bool merge_predicate(type_t a_key, type_t b_key,
   merge_range_t range, comp_t comp) {
-  if(range_check && !range.a_valid()) return false;
-  if(range_check && !range.b_valid()) return true;
+  if(range_check && range.a_begin >= range.a_end) return false;
+  if(range_check && range.b_begin >= range.b_end) return true;
   return (bounds_upper == bounds) ? comp(a_key, b_key) : !comp(b_key, a_key);
 }
 

@@ -1,6 +1,7 @@
-// mgpu for AMD CDNA4: interval expand / gather / scatter / move, all thin
-// functors over transform_lbs (interface after
-// src/moderngpu/kernel_intervalmove.hxx:7-65).
+// mgpu for AMD CDNA4: the interval functions.  Each is transform_lbs with a
+// functor that copies one item; the per-segment values (fill value, gather
+// base, scatter base) travel as the cached tuple.  Signatures after
+// src/moderngpu/kernel_intervalmove.hxx:7-65.
 #pragma once
 #include "kernel_load_balance.hxx"
 
@@ -35,68 +36,73 @@ struct interval_expand_f<type_t, type_t*> {
     store_consecutive<W>(output + index, x);
   }
 };
+
+// One item of gather / scatter / move.  The segment's tuple holds the scatter
+// base (if scattering) followed by the gather base (if gathering); an item
+// that is neither gathered nor scattered sits at its own index.
+template<bool scatters, bool gathers, typename input_it, typename output_it>
+struct interval_copy_f {
+  input_it input;
+  output_it output;
+  template<typename bases_t>
+  MGPU_DEVICE void operator()(int index, int, int rank, bases_t bases) const {
+    int from = index, to = index;
+    if constexpr(scatters) to = get<0>(bases) + rank;
+    if constexpr(gathers) from = get<scatters ? 1 : 0>(bases) + rank;
+    output[to] = input[from];
+  }
+};
+
 } // namespace detail
 
-// output[index] = input[segment of index]: each per-segment value is
-// replicated over the segment's items.
+// Segment s's one value written to each of its items:
+// output[i] = input[segment of i].
 template<typename launch_arg_t = empty_t, typename input_it,
   typename segments_it, typename output_it>
 void interval_expand(input_it input, int count, segments_it segments,
   int num_segments, output_it output, context_t& context) {
-
   typedef typename std::iterator_traits<input_it>::value_type type_t;
-  transform_lbs<launch_arg_t>(
-    detail::interval_expand_f<type_t, output_it> { output },
-    count, segments, num_segments, make_tuple(input), context);
+  detail::interval_expand_f<type_t, output_it> fill { output };
+  transform_lbs<launch_arg_t>(fill, count, segments, num_segments,
+    make_tuple(input), context);
 }
 
-// output[index] = input[gather[seg] + rank].
+// Segment s reads its items from input starting at gather[s]:
+// output[i] = input[gather[s] + rank of i].
 template<typename launch_arg_t = empty_t, typename input_it,
   typename segments_it, typename gather_it, typename output_it>
 void interval_gather(input_it input, int count, segments_it segments,
   int num_segments, gather_it gather, output_it output, context_t& context) {
-
-  transform_lbs<launch_arg_t>(
-    []MGPU_DEVICE(int index, int, int rank, tuple<int> desc,
-      input_it input, output_it output) {
-      output[index] = input[get<0>(desc) + rank];
-    },
-    count, segments, num_segments, make_tuple(gather), context, input, output
-  );
+  detail::interval_copy_f<false, true, input_it, output_it> copy {
+    input, output };
+  transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
+    make_tuple(gather), context);
 }
 
-// output[scatter[seg] + rank] = input[index].
+// Segment s writes its items to output starting at scatter[s]:
+// output[scatter[s] + rank of i] = input[i].
 template<typename launch_arg_t = empty_t, typename input_it,
   typename segments_it, typename scatter_it, typename output_it>
 void interval_scatter(input_it input, int count, segments_it segments,
   int num_segments, scatter_it scatter, output_it output,
   context_t& context) {
-
-  transform_lbs<launch_arg_t>(
-    []MGPU_DEVICE(int index, int, int rank, tuple<int> desc,
-      input_it input, output_it output) {
-      output[get<0>(desc) + rank] = input[index];
-    },
-    count, segments, num_segments, make_tuple(scatter), context, input, output
-  );
+  detail::interval_copy_f<true, false, input_it, output_it> copy {
+    input, output };
+  transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
+    make_tuple(scatter), context);
 }
 
-// output[scatter[seg] + rank] = input[gather[seg] + rank].
+// Both at once: output[scatter[s] + rank] = input[gather[s] + rank].
 template<typename launch_arg_t = empty_t,
   typename input_it, typename segments_it, typename scatter_it,
   typename gather_it, typename output_it>
 void interval_move(input_it input, int count, segments_it segments,
   int num_segments, scatter_it scatter, gather_it gather, output_it output,
   context_t& context) {
-
-  transform_lbs<launch_arg_t>(
-    []MGPU_DEVICE(int, int, int rank, tuple<int, int> desc,
-      input_it input, output_it output) {
-      output[get<0>(desc) + rank] = input[get<1>(desc) + rank];
-    },
-    count, segments, num_segments, make_tuple(scatter, gather), context,
-    input, output
-  );
+  detail::interval_copy_f<true, true, input_it, output_it> copy {
+    input, output };
+  transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
+    make_tuple(scatter, gather), context);
 }
 
 END_MGPU_NAMESPACE

@@ -145,7 +145,7 @@ enum { lbs_phase_partition = 1, lbs_phase_tiles = 2, lbs_phase_all = 3 };
 
 // Ints of partition storage for `total` merged elements cut into tiles of nv:
 // one (items, starts) pair per split.
-MGPU_HOST_DEVICE inline size_t lbs_partition_ints(int total, int nv) {
+MGPU_HOST_DEVICE size_t lbs_partition_ints(int total, int nv) {
   return 2 * ((size_t)div_up(total, lbs_tile_spacing(nv)) + 1);
 }
 

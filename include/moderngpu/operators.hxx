@@ -52,117 +52,111 @@ MGPU_DEF_BINARY(minimum_t, type_t, mgpu::min(a, b))
 #undef MGPU_DEF_BINARY
 
 ////////////////////////////////////////////////////////////////////////////////
-// CRTP bases for index-addressed iterators.  outer_t supplies
-// value_type operator()(int_t index).
+// Iterators that compute their values from an index instead of reading memory.
+// They offer what the library's kernels use of a random-access iterator:
+// it[i], *it, it + n, it - n, it += n, it -= n and the iterator_traits types.
 
+// The four offset operators for a class self_t whose position is `member`.
+#define MGPU_ITERATOR_OFFSETS(self_t, int_t, member)                          \
+  MGPU_HOST_DEVICE self_t& operator+=(int_t n) {                              \
+    member += n; return static_cast<self_t&>(*this);                          \
+  }                                                                           \
+  MGPU_HOST_DEVICE self_t& operator-=(int_t n) {                              \
+    member -= n; return static_cast<self_t&>(*this);                          \
+  }                                                                           \
+  MGPU_HOST_DEVICE self_t operator+(int_t n) const {                          \
+    self_t moved = static_cast<const self_t&>(*this);                         \
+    moved.member += n; return moved;                                          \
+  }                                                                           \
+  MGPU_HOST_DEVICE self_t operator-(int_t n) const {                          \
+    self_t moved = static_cast<const self_t&>(*this);                         \
+    moved.member -= n; return moved;                                          \
+  }
+
+// CRTP base: a position and the offset operators.
 template<typename outer_t, typename int_t, typename value_type>
-struct iterator_t : public std::iterator_traits<const value_type*> {
+struct iterator_t : std::iterator_traits<const value_type*> {
   int_t index;
-
   iterator_t() = default;
   MGPU_HOST_DEVICE iterator_t(int_t i) : index(i) { }
-
-  MGPU_HOST_DEVICE outer_t& operator+=(int_t diff) {
-    index += diff;
-    return *static_cast<outer_t*>(this);
-  }
-  MGPU_HOST_DEVICE outer_t& operator-=(int_t diff) {
-    index -= diff;
-    return *static_cast<outer_t*>(this);
-  }
-  MGPU_HOST_DEVICE outer_t operator+(int_t diff) const {
-    outer_t cp = *static_cast<const outer_t*>(this);
-    cp.index += diff;
-    return cp;
-  }
-  MGPU_HOST_DEVICE outer_t operator-(int_t diff) const {
-    outer_t cp = *static_cast<const outer_t*>(this);
-    cp.index -= diff;
-    return cp;
-  }
+  MGPU_ITERATOR_OFFSETS(outer_t, int_t, index)
 };
 
+// CRTP base of the read-only ones: outer_t::operator()(position) is the value.
 template<typename outer_t, typename int_t, typename value_type>
-struct const_iterator_t : public iterator_t<outer_t, int_t, value_type> {
-  typedef iterator_t<outer_t, int_t, value_type> base_t;
-
+struct const_iterator_t : iterator_t<outer_t, int_t, value_type> {
   const_iterator_t() = default;
-  MGPU_HOST_DEVICE const_iterator_t(int_t i) : base_t(i) { }
+  MGPU_HOST_DEVICE const_iterator_t(int_t i) :
+    iterator_t<outer_t, int_t, value_type>(i) { }
 
-  MGPU_HOST_DEVICE value_type operator[](int_t diff) const {
-    return static_cast<const outer_t&>(*this)(base_t::index + diff);
+  MGPU_HOST_DEVICE value_type operator[](int_t n) const {
+    return static_cast<const outer_t&>(*this)(this->index + n);
   }
-  MGPU_HOST_DEVICE value_type operator*() const {
-    return (*this)[0];
-  }
+  MGPU_HOST_DEVICE value_type operator*() const { return (*this)[0]; }
 };
 
-// Store iterator that drops what is written to it.
+// Accepts any store and keeps nothing (an unwanted output of a function that
+// produces several).
 template<typename value_type>
 struct discard_iterator_t :
   iterator_t<discard_iterator_t<value_type>, int, value_type> {
-
   struct assign_t {
-    MGPU_HOST_DEVICE value_type operator=(value_type) {
-      return value_type();
-    }
+    MGPU_HOST_DEVICE value_type operator=(value_type) { return value_type(); }
   };
   MGPU_HOST_DEVICE assign_t operator[](int) const { return assign_t(); }
   MGPU_HOST_DEVICE assign_t operator*() const { return assign_t(); }
 };
 
-// it[i] == (type_t)(base + i).  load_balance_partitions merges this against
-// the segment starts (reference search.hxx:35).
+// it[i] is (type_t)(start + i): the item indices that
+// load_balance_partitions merges with the segment starts
+// (src/moderngpu/search.hxx:35).
 template<typename type_t, typename int_t = int>
 struct counting_iterator_t :
   const_iterator_t<counting_iterator_t<type_t>, int_t, type_t> {
-
+  typedef const_iterator_t<counting_iterator_t<type_t>, int_t, type_t> base_t;
   counting_iterator_t() = default;
-  MGPU_HOST_DEVICE counting_iterator_t(type_t i) :
-    const_iterator_t<counting_iterator_t, int_t, type_t>(i) { }
-
-  MGPU_HOST_DEVICE type_t operator()(int_t index) const {
-    return (type_t)index;
-  }
+  MGPU_HOST_DEVICE counting_iterator_t(type_t start) : base_t(start) { }
+  MGPU_HOST_DEVICE type_t operator()(int_t at) const { return (type_t)at; }
 };
 
-// it[i] == offset + i * stride.
+// it[i] is offset + i * stride.
 template<typename type_t, typename int_t = int>
 struct strided_iterator_t :
   const_iterator_t<strided_iterator_t<type_t>, int_t, int> {
-
+  typedef const_iterator_t<strided_iterator_t<type_t>, int_t, int> base_t;
   type_t offset, stride;
-
   strided_iterator_t() = default;
   MGPU_HOST_DEVICE strided_iterator_t(type_t offset_, type_t stride_) :
-    const_iterator_t<strided_iterator_t, int_t, type_t>(0),
-    offset(offset_), stride(stride_) { }
-
-  MGPU_HOST_DEVICE type_t operator()(int_t index) const {
-    return offset + index * stride;
+    base_t(0), offset(offset_), stride(stride_) { }
+  MGPU_HOST_DEVICE type_t operator()(int_t at) const {
+    return offset + at * stride;
   }
 };
 
-// it[i] == value.
+// it[i] is value for every i.
 template<typename type_t>
 struct constant_iterator_t :
   const_iterator_t<constant_iterator_t<type_t>, int, type_t> {
-
+  typedef const_iterator_t<constant_iterator_t<type_t>, int, type_t> base_t;
   type_t value;
-
   MGPU_HOST_DEVICE constant_iterator_t(type_t value_) :
-    const_iterator_t<constant_iterator_t, int, type_t>(0), value(value_) { }
-
+    base_t(0), value(value_) { }
   MGPU_HOST_DEVICE type_t operator()(int) const { return value; }
 };
 
 ////////////////////////////////////////////////////////////////////////////////
-// lambda_iterator_t wraps a load functor f(index)->value and/or a store
-// functor g(value, index).  transform_segreduce feeds segreduce through
-// make_load_iterator (reference kernel_segreduce.hxx:278).
+// lambda_iterator_t: it[i] calls load(i) when read and store(x, i) when
+// assigned to.  Either functor may be empty_t, which makes that direction a
+// compile-time error.  transform_segreduce and transform_scan feed their
+// kernels through make_load_iterator (src/moderngpu/kernel_segreduce.hxx:278).
 
 template<typename load_t, typename store_t, typename value_type, typename int_t>
 struct lambda_iterator_t : std::iterator_traits<const value_type*> {
+  enum {
+    can_load = !std::is_same<load_t, empty_t>::value,
+    can_store = !std::is_same<store_t, empty_t>::value
+  };
+
   load_t load;
   store_t store;
   int_t base;
@@ -170,59 +164,38 @@ struct lambda_iterator_t : std::iterator_traits<const value_type*> {
   lambda_iterator_t(load_t load_, store_t store_, int_t base_) :
     load(load_), store(store_), base(base_) { }
 
-  // Proxy returned by operator[]: converts to the value (load) or accepts an
-  // assignment (store).
+  // What it[i] returns: reads as the value, takes an assignment.
   struct assign_t {
     load_t load;
     store_t store;
     int_t index;
 
-    MGPU_LAMBDA assign_t& operator=(value_type rhs) {
-      static_assert(!std::is_same<store_t, empty_t>::value,
-        "load_iterator is being stored to.");
-      store(rhs, index);
-      return *this;
-    }
     MGPU_LAMBDA operator value_type() const {
-      static_assert(!std::is_same<load_t, empty_t>::value,
-        "store_iterator is being loaded from.");
+      static_assert(can_load, "store_iterator is being loaded from.");
       return load(index);
+    }
+    MGPU_LAMBDA assign_t& operator=(value_type x) {
+      static_assert(can_store, "load_iterator is being stored to.");
+      store(x, index);
+      return *this;
     }
   };
 
-  MGPU_LAMBDA assign_t operator[](int_t index) const {
-    return assign_t { load, store, base + index };
+  MGPU_LAMBDA assign_t operator[](int_t n) const {
+    return assign_t { load, store, base + n };
   }
-  MGPU_LAMBDA assign_t operator*() const {
-    return assign_t { load, store, base };
-  }
+  MGPU_LAMBDA assign_t operator*() const { return (*this)[0]; }
 
-  MGPU_HOST_DEVICE lambda_iterator_t& operator+=(int_t offset) {
-    base += offset;
-    return *this;
-  }
-  MGPU_HOST_DEVICE lambda_iterator_t& operator-=(int_t offset) {
-    base -= offset;
-    return *this;
-  }
-  MGPU_HOST_DEVICE lambda_iterator_t operator+(int_t offset) const {
-    lambda_iterator_t cp = *this;
-    cp.base += offset;
-    return cp;
-  }
-  MGPU_HOST_DEVICE lambda_iterator_t operator-(int_t offset) const {
-    lambda_iterator_t cp = *this;
-    cp.base -= offset;
-    return cp;
-  }
+  MGPU_ITERATOR_OFFSETS(lambda_iterator_t, int_t, base)
 };
+#undef MGPU_ITERATOR_OFFSETS
 
+// Placeholders for a direction that is not used but must exist.
 template<typename value_type>
 struct trivial_load_functor {
   template<typename int_t>
   MGPU_HOST_DEVICE value_type operator()(int_t) const { return value_type(); }
 };
-
 template<typename value_type>
 struct trivial_store_functor {
   template<typename int_t>
@@ -231,22 +204,19 @@ struct trivial_store_functor {
 
 template<typename value_type, typename int_t = int, typename load_t,
   typename store_t>
-lambda_iterator_t<load_t, store_t, value_type, int_t>
-make_load_store_iterator(load_t load, store_t store, int_t base = 0) {
+auto make_load_store_iterator(load_t load, store_t store, int_t base = 0) {
   return lambda_iterator_t<load_t, store_t, value_type, int_t>(
     load, store, base);
 }
-
 template<typename value_type, typename int_t = int, typename load_t>
-lambda_iterator_t<load_t, empty_t, value_type, int_t>
-make_load_iterator(load_t load, int_t base = 0) {
-  return make_load_store_iterator<value_type>(load, empty_t(), base);
+auto make_load_iterator(load_t load, int_t base = 0) {
+  return lambda_iterator_t<load_t, empty_t, value_type, int_t>(
+    load, empty_t(), base);
 }
-
 template<typename value_type, typename int_t = int, typename store_t>
-lambda_iterator_t<empty_t, store_t, value_type, int_t>
-make_store_iterator(store_t store, int_t base = 0) {
-  return make_load_store_iterator<value_type>(empty_t(), store, base);
+auto make_store_iterator(store_t store, int_t base = 0) {
+  return lambda_iterator_t<empty_t, store_t, value_type, int_t>(
+    empty_t(), store, base);
 }
 
 END_MGPU_NAMESPACE

@@ -1,29 +1,23 @@
-// mgpu for AMD CDNA4: printf into a std::string (used by device_prop_string).
+// mgpu for AMD CDNA4: formatted text into a std::string, for the device
+// description that standard_context_t prints (the helper has the name it has
+// in src/moderngpu/util.hxx:11).
 #pragma once
-#include "types.hxx"
-#include <cstdarg>
 #include <cstdio>
 #include <string>
-#include <vector>
+#include "types.hxx"
 
 BEGIN_MGPU_NAMESPACE
-
 namespace detail {
 
-inline std::string stringprintf(const char* format, ...) {
-  va_list args;
-  va_start(args, format);
-  int len = vsnprintf(nullptr, 0, format, args);
-  va_end(args);
-  if(len <= 0) return std::string();
-
-  std::vector<char> buffer(len + 1);
-  va_start(args, format);
-  vsnprintf(buffer.data(), buffer.size(), format, args);
-  va_end(args);
-  return std::string(buffer.data(), len);
+// snprintf twice: once for the length, once into a string of that length.
+template<typename... args_t>
+std::string stringprintf(const char* format, args_t... args) {
+  int length = std::snprintf(nullptr, 0, format, args...);
+  std::string text(length > 0 ? length : 0, '\0');
+  if(length > 0)
+    std::snprintf(&text[0], (size_t)length + 1, format, args...);
+  return text;
 }
 
 } // namespace detail
-
 END_MGPU_NAMESPACE

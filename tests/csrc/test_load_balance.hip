@@ -1,32 +1,47 @@
-// Caller shaped like the reference's load-balancing-search test (moderngpu
-// tests/test_load_balance.cu): segment starts every `spacing` items,
-// load_balance_search, expect lbs[i] == i / spacing.  Non-zero exit on error.
+// A C++ caller of load_balance_search with the reference's own test shape
+// (moderngpu tests/test_load_balance.cu: 200030 items, a segment start every
+// 100 items) plus a few more (count, spacing) pairs around tile edges.
+// Expected segment of item i is floor(i / spacing), checked here with a
+// running counter rather than a division.  Exit status 1 on the first
+// mismatch.
 #include <moderngpu/kernel_load_balance.hxx>
 #include <cstdio>
 
-using namespace mgpu;
+static bool check_even_segments(int count, int spacing,
+  mgpu::context_t& context) {
+  int num_segments = mgpu::div_up(count, spacing);
+  std::vector<int> starts;
+  for(int s = 0; s < num_segments; ++s) starts.push_back(s * spacing);
 
-int main() {
-  standard_context_t context(false);
+  mgpu::mem_t<int> segments = mgpu::to_mem(starts, context);
+  mgpu::mem_t<int> found(count, context);
+  mgpu::load_balance_search(count, segments.data(), num_segments,
+    found.data(), context);
 
-  int count = 200030;
-  int spacing = 100;
-  int num_segments = div_up(count, spacing);
-  std::vector<int> segments_host(num_segments);
-  for(int i = 0; i < num_segments; ++i) segments_host[i] = i * spacing;
-  mem_t<int> segments = to_mem(segments_host, context);
-
-  mem_t<int> lbs(count, context);
-  load_balance_search(count, segments.data(), num_segments, lbs.data(),
-    context);
-
-  std::vector<int> lbs_host = from_mem(lbs);
-  for(size_t i = 0; i < lbs_host.size(); ++i) {
-    if(lbs_host[i] != (int)i / spacing) {
-      printf("ERROR AT %d: %d\n", (int)i, lbs_host[i]);
-      return 1;
+  std::vector<int> host = mgpu::from_mem(found);
+  int expected = 0, left = spacing;
+  for(int i = 0; i < count; ++i, --left) {
+    if(!left) { ++expected; left = spacing; }
+    if(host[i] != expected) {
+      printf("count %d spacing %d: item %d in segment %d, expected %d\n",
+        count, spacing, i, host[i], expected);
+      return false;
     }
   }
-  printf("load_balance_search: %d items passed\n", count);
+  return true;
+}
+
+int main() {
+  mgpu::standard_context_t context(false);
+  const int cases[][2] = {
+    { 200030, 100 }, { 200030, 1 }, { 6144, 6144 }, { 6145, 7 },
+    { 1000003, 4099 }
+  };
+  int items = 0;
+  for(const int (&c)[2] : cases) {
+    if(!check_even_segments(c[0], c[1], context)) return 1;
+    items += c[0];
+  }
+  printf("load_balance_search: %d items passed\n", items);
   return 0;
 }
