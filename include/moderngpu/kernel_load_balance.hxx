@@ -149,6 +149,24 @@ MGPU_HOST_DEVICE size_t lbs_partition_ints(int total, int nv) {
   return 2 * ((size_t)div_up(total, lbs_tile_spacing(nv)) + 1);
 }
 
+// Cuts the merge of `count` items with the segment starts into tiles of at
+// most nv elements and writes the splits as pairs (lbs_partition_ints ints).
+// Returns the number of tiles.
+template<typename segments_it>
+int lbs_partition_tiles(int count, segments_it segments, int num_segments,
+  int nv, int* pairs, context_t& context) {
+  int spacing = lbs_tile_spacing(nv);
+  // A tile too small to give up lbs_snap_slack elements is cut at every nv
+  // exactly and its splits stay where they fall.
+  if(spacing < nv)
+    load_balance_partitions_snapped<lbs_snap_items, lbs_snap_window>(count,
+      segments, num_segments, spacing, pairs, context);
+  else
+    load_balance_partitions_snapped<1, 1>(count, segments, num_segments,
+      spacing, pairs, context);
+  return div_up(count + num_segments, spacing);
+}
+
 // Partition + tile kernels with the partition array in caller-provided
 // device memory: lbs_partition_ints(count + num_segments, nv) ints.
 template<typename launch_t, typename func_t, typename segments_it,
@@ -158,13 +176,12 @@ void transform_lbs_launch(func_t f, int count, segments_it segments,
   context_t& context, args_t... args) {
 
   if(count + num_segments <= 0) return;
-  int spacing = lbs_tile_spacing(launch_t::nv(context));
+  int nv = launch_t::nv(context);
   if(phases & lbs_phase_partition)
-    load_balance_partitions_snapped<lbs_snap_items, lbs_snap_window>(count,
-      segments, num_segments, spacing, mp_data, context);
+    lbs_partition_tiles(count, segments, num_segments, nv, mp_data, context);
 
   if(phases & lbs_phase_tiles) {
-    int num_tiles = div_up(count + num_segments, spacing);
+    int num_tiles = div_up(count + num_segments, lbs_tile_spacing(nv));
     transform_lbs_f<launch_t, func_t, segments_it, pointers_t, int>
       k { f, count, segments, num_segments, caching_iterators, mp_data,
         num_tiles };

@@ -1,0 +1,388 @@
+// mgpu for AMD CDNA4: dynamic work creation on top of the load-balancing
+// search.  Every work-item of a segmented workload may create a segment of
+// new work-items for the next pass (a vertex reached by a frontier edge
+// creates one work-item per outgoing edge, say):
+//
+//   auto engine = expt::lbs_workcreate(count, segments, num_segments, context);
+//   auto sizes = engine.upsweep(f, cached);    f(index, seg, rank, tuple)
+//   mem_t<int> next = engine.downsweep(g, cached, args...);
+//                                    g(dest_seg, index, seg, rank, tuple, args...)
+//
+// upsweep calls f once per work-item; an item that returns n > 0 creates a
+// segment of n new work-items.  It returns how many segments and work-items
+// the next pass has, so the caller can allocate per-segment outputs.
+// downsweep calls g once per creating item, in item order, with the number of
+// the segment it creates; g returns the same count f did and may store
+// whatever describes the new segment.  The result holds the start offsets of
+// the new segments.  Interface after
+// src/moderngpu/kernel_workcreate.hxx:14-268.
+//
+// Both sweeps decode the same tiles (the engine owns the partition).  Between
+// them a thread keeps one bit per item it looked at; the position of a
+// creating item among all creating items comes from wavefront ballots: in a
+// row of nt consecutive items each wavefront owns 64 consecutive ones, so
+// popcounts per (row, wavefront), scanned over the tile, plus the popcount
+// of the lower lanes give the position without compacting anything through
+// LDS.  The start offsets come from the same table scheme over wave-level
+// prefix sums of the counts.
+#pragma once
+
+#include "kernel_load_balance.hxx"
+#include "kernel_scan.hxx"
+#include "cta_reduce.hxx"
+
+BEGIN_MGPU_NAMESPACE
+
+namespace expt {
+
+namespace detail {
+
+using namespace mgpu::detail;
+
+// 256 threads x 12 items: the callbacks gather from global memory, so more
+// resident CTAs per CU matter more here than the longest possible tile.
+typedef launch_box_t<arch_gfx950_cta<256, 12, 12> > workcreate_launch_default_t;
+
+template<typename arg_t>
+struct is_tuple_t : std::false_type { };
+template<typename... args_t>
+struct is_tuple_t<tuple<args_t...> > : std::true_type { };
+
+// Totals of a tile, and after the scan its offsets, as one 64-bit sum:
+// creating items in the low word, created work-items in the high word.
+// Neither total reaches 2^31, so the low word never carries into the high.
+typedef unsigned long long tile_total_t;
+MGPU_HOST_DEVICE tile_total_t pack_total(int creators, int work) {
+  return (tile_total_t)(unsigned)work << 32 | (unsigned)creators;
+}
+MGPU_HOST_DEVICE int total_creators(tile_total_t x) {
+  return (int)(unsigned)x;
+}
+MGPU_HOST_DEVICE int total_work(tile_total_t x) { return (int)(x >> 32); }
+
+// What the two kernels share: tile decode and per-item (seg, rank, cached).
+template<typename launch_t, typename segments_it, typename pointers_t>
+struct workcreate_tile_t {
+  typedef typename launch_t::sm_ptx params_t;
+  enum {
+    nt = params_t::nt, vt = params_t::vt, num_waves = nt / warp_size,
+    table_size = vt * num_waves
+  };
+  static_assert(0 == nt % warp_size, "whole wavefronts only");
+  static_assert(vt <= 32, "one bit per item in a 32-bit word");
+  static_assert(table_size <= nt, "the per-row table is scanned by one CTA scan");
+
+  typedef cta_load_balance_t<nt, vt> load_balance_t;
+  typedef typename load_balance_t::layout_t layout_t;
+  typedef cached_segment_load_t<nt, pointers_t> cached_load_t;
+  typedef typename cached_load_t::value_t value_t;
+  typedef cta_scan_t<nt, int> scan_t;
+  typedef cta_reduce_t<nt, tile_total_t> reduce_t;
+
+  struct storage_t {
+    typename load_balance_t::storage_t lbs;
+    typename cached_load_t::storage_t cached;
+    union {
+      typename scan_t::storage_t scan;
+      typename reduce_t::storage_t reduce;
+    };
+    int table[table_size];
+    MGPU_DEVICE storage_t() { }
+  };
+
+  int count;
+  segments_it segments;
+  int num_segments;
+  pointers_t caching_iterators;
+  const int* pairs;
+  int num_tiles;
+
+  // After decode(): visit(i, index, seg, rank, cached) for the items of the
+  // tile this thread owns, item nt * i + tid in step i.
+  struct decoded_t {
+    merge_range_t range;
+    bool staged;
+  };
+  MGPU_DEVICE decoded_t decode(int tid, int tile, storage_t& shared) const {
+    merge_range_t range = paired_tile_range(count, num_segments, tile,
+      load_balance_t::nv, pairs);
+    load_balance_t().fill(range, segments, tid, shared.lbs);
+    bool staged = cached_load_t::stage(tid, range.b_begin - 1,
+      range.b_count() + 1, shared.cached, caching_iterators);
+    return decoded_t { range, staged };
+  }
+
+  template<typename visit_t>
+  MGPU_DEVICE void item(int i, int tid, const decoded_t& tile,
+    const storage_t& shared, visit_t visit) const {
+    int a_count = tile.range.a_count();
+    int seg_base = tile.range.b_begin - 1;
+    const int* slots = shared.lbs.indices;
+    const int* starts = slots + load_balance_t::starts_offset(a_count);
+    int p = nt * i + tid;
+    int rel = slots[layout_t::index(p)];
+    int seg = seg_base + rel;
+    int index = tile.range.a_begin + p;
+    visit(index, seg, index - starts[rel], cached_load_t::get(tile.staged,
+      rel, seg, shared.cached, caching_iterators));
+  }
+
+  // Exclusive scan of table[0 .. table_size) in place; entry
+  // num_waves * i + wave belongs to row i of wavefront `wave`, so the scan
+  // runs in item order.  Returns the total.
+  MGPU_DEVICE int scan_table(int tid, storage_t& shared) const {
+    __syncthreads();
+    int x = tid < table_size ? shared.table[tid] : 0;
+    scan_result_t<int> result = scan_t().scan(tid, x, shared.scan);
+    if(tid < table_size) shared.table[tid] = result.scan;
+    __syncthreads();
+    return result.reduction;
+  }
+};
+
+template<typename launch_t, typename func_t, typename segments_it,
+  typename pointers_t>
+struct workcreate_upsweep_f {
+  typedef workcreate_tile_t<launch_t, segments_it, pointers_t> tile_t;
+  typedef typename tile_t::value_t value_t;
+  enum { nt = tile_t::nt, vt = tile_t::vt };
+
+  tile_t tiles;
+  func_t f;
+  unsigned* bits_data;            // nt words per tile
+  tile_total_t* totals_data;      // one per tile
+
+  MGPU_DEVICE void operator()(int tid, int cta) const {
+    int tile = xcd_tile(cta, tiles.num_tiles);
+    if(tile >= tiles.num_tiles) return;
+    __shared__ typename tile_t::storage_t shared;
+    typename tile_t::decoded_t decoded = tiles.decode(tid, tile, shared);
+
+    unsigned bits = 0;
+    int work = 0;
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i) {
+      if(nt * i + tid < decoded.range.a_count()) {
+        tiles.item(i, tid, decoded, shared,
+          [&](int index, int seg, int rank, value_t cached) {
+            int created = f(index, seg, rank, cached);
+            if(created > 0) {
+              bits |= 1u << i;
+              work += created;
+            }
+          });
+      }
+    }
+    bits_data[nt * tile + tid] = bits;
+
+    tile_total_t total = typename tile_t::reduce_t().reduce(tid,
+      pack_total(popc(bits), work), shared.reduce, nt,
+      plus_t<tile_total_t>(), false);
+    if(!tid) totals_data[tile] = total;
+  }
+};
+
+template<typename launch_t, typename func_t, typename segments_it,
+  typename pointers_t>
+struct workcreate_downsweep_f {
+  typedef workcreate_tile_t<launch_t, segments_it, pointers_t> tile_t;
+  typedef typename tile_t::value_t value_t;
+  enum { nt = tile_t::nt, vt = tile_t::vt, num_waves = tile_t::num_waves };
+
+  tile_t tiles;
+  func_t f;
+  const unsigned* bits_data;
+  const tile_total_t* offsets_data;   // exclusive scan of the tile totals
+  int* segments_output;
+
+  template<typename... args_t>
+  MGPU_DEVICE void operator()(int tid, int cta, args_t... args) const {
+    int tile = xcd_tile(cta, tiles.num_tiles);
+    if(tile >= tiles.num_tiles) return;
+    __shared__ typename tile_t::storage_t shared;
+
+    int lane = tid % warp_size, wave = tid / warp_size;
+    unsigned bits = bits_data[nt * tile + tid];
+    tile_total_t offset = offsets_data[tile];
+
+    // Position of every creating item among the tile's creating items.
+    int below[vt];
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i) {
+      lanemask_t creators = ballot(0 != (bits & (1u << i)));
+      below[i] = popc(creators & lanemask_lt(lane));
+      if(!lane) shared.table[num_waves * i + wave] = popc(creators);
+    }
+    int num_creators = tiles.scan_table(tid, shared);
+    int dest[vt];
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i)
+      dest[i] = total_creators(offset) + shared.table[num_waves * i + wave] +
+        below[i];
+
+    // Tiles without a creating item have nothing to decode.  (The branch is
+    // uniform: every thread has the same num_creators.)
+    if(!num_creators) return;
+    typename tile_t::decoded_t decoded = tiles.decode(tid, tile, shared);
+
+    int created[vt];
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i) {
+      created[i] = 0;
+      if(bits & (1u << i)) {
+        tiles.item(i, tid, decoded, shared,
+          [&](int index, int seg, int rank, value_t cached) {
+            created[i] = max(0, (int)f(dest[i], index, seg, rank, cached,
+              args...));
+          });
+      }
+    }
+
+    // Start of every new segment: work-items created in front of it.
+    int before[vt];
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i) {
+      int inclusive = wave_scan(created[i], plus_t<int>(), lane);
+      before[i] = inclusive - created[i];
+      if(warp_size - 1 == lane)
+        shared.table[num_waves * i + wave] = inclusive;
+    }
+    tiles.scan_table(tid, shared);
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i) {
+      if(bits & (1u << i))
+        segments_output[dest[i]] = total_work(offset) +
+          shared.table[num_waves * i + wave] + before[i];
+    }
+  }
+};
+
+} // namespace detail
+
+template<typename launch_arg_t, typename segments_it>
+struct workcreate_t {
+  typedef typename conditional_typedef_t<launch_arg_t,
+    detail::workcreate_launch_default_t>::type_t launch_t;
+  typedef detail::tile_total_t tile_total_t;
+
+  int count;
+  segments_it segments;
+  int num_segments;
+  context_t& context;
+
+  cta_dim_t cta_dim;
+  int num_tiles;
+
+  mem_t<int> pairs;               // splits, (items, starts) per tile end
+  mem_t<unsigned> bits;           // per thread and tile: who creates work
+  mem_t<tile_total_t> offsets;    // per tile: creators and work in front
+  tile_total_t total;
+
+  // Sizes of the next pass.
+  struct count_t {
+    int count;                    // work-items created
+    int num_segments;             // items that created any
+  };
+
+  workcreate_t(int count_, segments_it segments_, int num_segments_,
+    context_t& context_) : count(count_), segments(segments_),
+    num_segments(num_segments_), context(context_), total(0) {
+
+    cta_dim = launch_t::cta_dim(context);
+    int nv = cta_dim.nv();
+    int64_t merged = (int64_t)count + num_segments;
+    if(count < 0 || num_segments < 0 || merged >= ((int64_t)1 << 31))
+      throw cuda_exception_t(hipErrorInvalidValue);
+    num_tiles = 0;
+    if(!merged) return;
+
+    pairs = mem_t<int>(mgpu::detail::lbs_partition_ints((int)merged, nv),
+      context);
+    num_tiles = mgpu::detail::lbs_partition_tiles(count, segments,
+      num_segments, nv, pairs.data(), context);
+    bits = mem_t<unsigned>((size_t)num_tiles * cta_dim.nt, context);
+    offsets = mem_t<tile_total_t>(num_tiles, context);
+  }
+
+  // f(int index, int seg, int rank, tuple<...> cached) returns the number of
+  // work-items the item creates; zero or less creates nothing.  Waits for
+  // the device: the totals come back to the host.
+  template<typename func_t, typename pointers_t>
+  count_t upsweep(func_t f, pointers_t caching_iterators) {
+    if(!num_tiles) return count_t { 0, 0 };
+
+    typedef detail::workcreate_tile_t<launch_t, segments_it, pointers_t>
+      tile_t;
+    mem_t<tile_total_t> totals(num_tiles, context);
+    detail::workcreate_upsweep_f<launch_t, func_t, segments_it, pointers_t>
+      k { tile_t { count, segments, num_segments, caching_iterators,
+        pairs.data(), num_tiles }, f, bits.data(), totals.data() };
+    cta_launch<launch_t>(k, mgpu::detail::xcd_grid(num_tiles), context);
+
+    // Offsets of every tile; the grand total goes to pinned host memory and
+    // is there once the event has passed.
+    mem_t<tile_total_t> total_host(1, context, memory_space_host);
+    scan_event(totals.data(), num_tiles, offsets.data(),
+      plus_t<tile_total_t>(), total_host.data(), context, context.event());
+    hipError_t status = hipEventSynchronize(context.event());
+    if(hipSuccess != status) throw cuda_exception_t(status);
+
+    total = total_host.data()[0];
+    return count_t { detail::total_work(total),
+      detail::total_creators(total) };
+  }
+
+  // f(int index, int seg, int rank).
+  template<typename func_t>
+  count_t upsweep(func_t f) {
+    return upsweep([=]MGPU_DEVICE(int index, int seg, int rank, tuple<>) {
+      return f(index, seg, rank);
+    }, tuple<>());
+  }
+
+  // f(int dest_seg, int index, int seg, int rank, tuple<...> cached, args...)
+  // for every item that created work in the upsweep; dest_seg counts those
+  // items in item order.  f returns the count it returned in the upsweep.
+  // The result has one start offset per new segment.
+  template<typename func_t, typename pointers_t, typename... args_t,
+    typename = enable_if_t<detail::is_tuple_t<pointers_t>::value> >
+  mem_t<int> downsweep(func_t f, pointers_t caching_iterators,
+    args_t... args) {
+    int num_dest_segments = detail::total_creators(total);
+    mem_t<int> result(num_dest_segments, context);
+    if(!num_tiles || !num_dest_segments) return result;
+
+    typedef detail::workcreate_tile_t<launch_t, segments_it, pointers_t>
+      tile_t;
+    detail::workcreate_downsweep_f<launch_t, func_t, segments_it, pointers_t>
+      k { tile_t { count, segments, num_segments, caching_iterators,
+        pairs.data(), num_tiles }, f, bits.data(), offsets.data(),
+        result.data() };
+    cta_launch<launch_t>(k, mgpu::detail::xcd_grid(num_tiles), context,
+      args...);
+    return result;
+  }
+
+  // f(int dest_seg, int index, int seg, int rank, args...).
+  template<typename func_t, typename... args_t>
+  mem_t<int> downsweep(func_t f, args_t... args) {
+    return downsweep(
+      [=]MGPU_DEVICE(int dest_seg, int index, int seg, int rank, tuple<>,
+        args_t... args) {
+        return f(dest_seg, index, seg, rank, args...);
+      }, tuple<>(), args...);
+  }
+};
+
+// One engine per pass: construct it, call upsweep, then downsweep.
+template<typename launch_arg_t = empty_t, typename segments_it>
+workcreate_t<launch_arg_t, segments_it>
+lbs_workcreate(int count, segments_it segments, int num_segments,
+  context_t& context) {
+  return workcreate_t<launch_arg_t, segments_it>(count, segments,
+    num_segments, context);
+}
+
+} // namespace expt
+
+END_MGPU_NAMESPACE

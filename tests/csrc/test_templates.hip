@@ -66,6 +66,25 @@ static int run_boxed(context_t& context) {
   return 0;
 }
 
+// load_balance_search under a caller's launch box, against the host merge.
+// Mean segment length 8: most tile boundaries have starts close behind them.
+template<typename launch_t>
+static int run_boxed_lbs(context_t& context) {
+  int count = 200003, num_segments = 25000;
+  std::vector<int> seg_host = make_segments(count, num_segments, 19);
+  mem_t<int> segments = to_mem(seg_host, context);
+  mem_t<int> found(count, context);
+  load_balance_search<launch_t>(count, segments.data(), num_segments,
+    found.data(), context);
+  std::vector<int> got = from_mem(found);
+  int seg = -1;
+  for(int i = 0; i < count; ++i) {
+    while(seg + 1 < num_segments && seg_host[seg + 1] <= i) ++seg;
+    CHECK(got[i] == seg);
+  }
+  return 0;
+}
+
 int main() {
   counting_context_t context;
 
@@ -80,6 +99,13 @@ int main() {
   CHECK(0 == run_boxed<box_cuda_t>(context));
   CHECK(0 == (run_boxed<launch_params_t<64, 5> >(context)));
   CHECK(0 == run_boxed<empty_t>(context));
+  // The search with tiles from 64 to 896 elements.
+  CHECK(0 == run_boxed_lbs<box_cuda_t>(context));
+  CHECK(0 == (run_boxed_lbs<launch_params_t<64, 1> >(context)));
+  CHECK(0 == (run_boxed_lbs<launch_params_t<64, 4> >(context)));
+  CHECK(0 == (run_boxed_lbs<launch_params_t<64, 5> >(context)));
+  CHECK(0 == (run_boxed_lbs<launch_params_t<128, 3> >(context)));
+  CHECK(0 == (run_boxed_lbs<launch_params_t<256, 2> >(context)));
   CHECK(context.allocs > 0 && context.frees > 0);
 
   // 2. user value type + user operator through segreduce.
