@@ -298,7 +298,45 @@ def make_scan(copies, kind):
     return wk
 
 
+def make_workcreate(copies):
+    """The step behind the path: 2^26 work-items in 2^20 segments (the segments
+    of configs[1]), a quarter of them creating 1..8 new work-items each."""
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    from oracle import oracle
+    w = workloads.config2()
+    n, s = w["values"].size, w["segments"].size
+    rng = np.random.Generator(np.random.PCG64(42))
+    host = rng.integers(1, 9, size=n, dtype=np.int32)
+    host[rng.random(n) >= 0.25] = 0
+    created = [_dev(host) for _ in range(copies)]
+    segs = [_dev(w["segments"]) for _ in range(copies)]
+    k = int(np.count_nonzero(host))
+    wk = Workload()
+    wk.key, wk.dtype = "workcreate_i32", "i32"
+    wk.name = ("lbs_workcreate upsweep + downsweep, 2^26 items in 2^20 segments, "
+               "%d items create work" % k)
+    wk.items = n
+    # upsweep: counts + starts in; downsweep: starts + the creators' counts in,
+    # four ints per new segment out.
+    wk.bytes = n * 4 + s * 4 + s * 4 + k * 4 + k * 16
+    wk.kernel = "workcreate upsweep + totals scan + downsweep (whole call, one host wait)"
+    wk.step = lambda i: m.workcreate(created[i % copies], segs[i % copies])
+    wk.tiles = wk.step
+
+    def check():
+        got = wk.step(0)
+        want = oracle.workcreate(host, w["segments"])
+        return got[0] == want[0] and all(
+            np.array_equal(g.cpu().numpy(), x) for g, x in zip(got[1:], want[1:]))
+    wk.check = check
+    wk.cpu = lambda: (lambda: oracle.workcreate(host, w["segments"]))
+    return wk
+
+
 FACTORIES = {
+    "workcreate_i32": make_workcreate,
     "scan_i32": lambda c: make_scan(c, "scan"),
     "reduce_f32": lambda c: make_scan(c, "reduce"),
     "c1_segreduce_i32": make_c1,

@@ -217,6 +217,39 @@ MGPU_HIP_API int mgpu_hip_reduce(const void* input, int count,
   void* reduction, int dtype, int op, void* workspace,
   size_t workspace_bytes, mgpu_stream_t stream);
 
+/* ---- dynamic work creation (the step after the search) ------------------ */
+
+/* mgpu::expt::lbs_workcreate (kernel_workcreate.hxx:14-268) with the counts
+ * read from an array: item i of a segmented workload creates a segment of
+ * created[i] new work-items (none if created[i] <= 0).  Arbitrary functors
+ * and cached iterators need the C++ templates.
+ *
+ * Bytes of workspace the two calls below share; the downsweep reads what the
+ * upsweep left there. */
+MGPU_HIP_API size_t mgpu_hip_workcreate_workspace_bytes(int count,
+  int num_segments);
+
+/* workcreate_t::upsweep (kernel_workcreate.hxx:64-145): stores
+ * sizes[0] = number of creating items (the new num_segments) and
+ * sizes[1] = sum of their counts (the new count).  sizes is 8-byte aligned
+ * device memory, or host memory the device can write; it is valid once the
+ * stream has reached this point. */
+MGPU_HIP_API int mgpu_hip_workcreate_upsweep(const int* created, int count,
+  const int* segments, int num_segments, int* sizes, void* workspace,
+  size_t workspace_bytes, mgpu_stream_t stream);
+
+/* workcreate_t::downsweep (kernel_workcreate.hxx:149-247), after an upsweep
+ * with the same arguments and workspace.  For the k-th creating item (in item
+ * order) stores new_segments[k] = sum of the counts of the creating items in
+ * front of it, and what the reference hands its downsweep functor:
+ * source_index[k] = the item, source_seg[k] = its segment, source_rank[k] =
+ * its rank in that segment.  Arrays of sizes[0] ints; the source_* ones may
+ * be NULL. */
+MGPU_HIP_API int mgpu_hip_workcreate_downsweep(const int* created, int count,
+  const int* segments, int num_segments, int* new_segments,
+  int* source_index, int* source_seg, int* source_rank, void* workspace,
+  size_t workspace_bytes, mgpu_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -18,13 +18,14 @@
 // src/moderngpu/kernel_workcreate.hxx:14-268.
 //
 // Both sweeps decode the same tiles (the engine owns the partition).  Between
-// them a thread keeps one bit per item it looked at; the position of a
-// creating item among all creating items comes from wavefront ballots: in a
-// row of nt consecutive items each wavefront owns 64 consecutive ones, so
-// popcounts per (row, wavefront), scanned over the tile, plus the popcount
-// of the lower lanes give the position without compacting anything through
-// LDS.  The start offsets come from the same table scheme over wave-level
-// prefix sums of the counts.
+// them a thread keeps one bit per item it looked at.  The downsweep finds the
+// position of a creating item among the tile's creating items from wavefront
+// ballots -- in a row of nt consecutive items each wavefront owns 64
+// consecutive ones, so popcounts per (row, wavefront), scanned over the tile,
+// plus the popcount of the lower lanes give it -- and gathers the creating
+// items in that order, so the calls run with all lanes busy and what they
+// store per new segment is contiguous.  The start offsets come from the same
+// table scheme over wave-level prefix sums of the counts.
 #pragma once
 
 #include "kernel_load_balance.hxx"
@@ -78,6 +79,8 @@ struct workcreate_tile_t {
   typedef typename cached_load_t::value_t value_t;
   typedef cta_scan_t<nt, int> scan_t;
   typedef cta_reduce_t<nt, tile_total_t> reduce_t;
+  typedef typename std::conditional<(nt * vt <= 65536), unsigned short,
+    int>::type target_t;
 
   struct storage_t {
     typename load_balance_t::storage_t lbs;
@@ -97,8 +100,6 @@ struct workcreate_tile_t {
   const int* pairs;
   int num_tiles;
 
-  // After decode(): visit(i, index, seg, rank, cached) for the items of the
-  // tile this thread owns, item nt * i + tid in step i.
   struct decoded_t {
     merge_range_t range;
     bool staged;
@@ -112,18 +113,61 @@ struct workcreate_tile_t {
     return decoded_t { range, staged };
   }
 
-  template<typename visit_t>
-  MGPU_DEVICE void item(int i, int tid, const decoded_t& tile,
-    const storage_t& shared, visit_t visit) const {
+  // Segment, rank and cached values of the thread's items, item nt * i + tid
+  // in position i.  Every LDS read is issued for every position, wanted or
+  // not, so that none of them waits behind a branch; a position outside
+  // `wanted` (bit i) gets the tile's first segment and values that mean
+  // nothing.  Cached values that are not staged in LDS are gathered from
+  // global memory for the wanted positions only.
+  struct items_t {
+    int seg[vt];
+    int rank[vt];
+    value_t cached[vt];
+  };
+  MGPU_DEVICE void items(int tid, const decoded_t& tile,
+    const storage_t& shared, unsigned wanted, items_t& x) const {
     int a_count = tile.range.a_count();
     int seg_base = tile.range.b_begin - 1;
     const int* slots = shared.lbs.indices;
     const int* starts = slots + load_balance_t::starts_offset(a_count);
-    int p = nt * i + tid;
+    int rel[vt];
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i) {
+      int p = nt * i + tid;
+      rel[i] = slots[layout_t::index(min(p, nt * vt - 1))];
+      if(p >= a_count) rel[i] = 0;
+    }
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i) {
+      x.seg[i] = seg_base + rel[i];
+      x.rank[i] = tile.range.a_begin + nt * i + tid - starts[rel[i]];
+    }
+    if(tile.staged) {
+      PRAGMA_UNROLL
+      for(int i = 0; i < vt; ++i)
+        x.cached[i] = cached_load_t::get(true, rel[i], x.seg[i],
+          shared.cached, caching_iterators);
+    } else {
+      PRAGMA_UNROLL
+      for(int i = 0; i < vt; ++i)
+        if(wanted & (1u << i))
+          x.cached[i] = cached_load_t::get(false, rel[i], x.seg[i],
+            shared.cached, caching_iterators);
+    }
+  }
+
+  // The same for the one item at tile position p < a_count:
+  // call(index, seg, rank, cached).
+  template<typename call_t>
+  MGPU_DEVICE void item(int p, const decoded_t& tile,
+    const storage_t& shared, call_t call) const {
+    const int* slots = shared.lbs.indices;
+    const int* starts = slots +
+      load_balance_t::starts_offset(tile.range.a_count());
     int rel = slots[layout_t::index(p)];
-    int seg = seg_base + rel;
+    int seg = tile.range.b_begin - 1 + rel;
     int index = tile.range.a_begin + p;
-    visit(index, seg, index - starts[rel], cached_load_t::get(tile.staged,
+    call(index, seg, index - starts[rel], cached_load_t::get(tile.staged,
       rel, seg, shared.cached, caching_iterators));
   }
 
@@ -158,19 +202,32 @@ struct workcreate_upsweep_f {
     __shared__ typename tile_t::storage_t shared;
     typename tile_t::decoded_t decoded = tiles.decode(tid, tile, shared);
 
+    // Bit i: item nt * i + tid exists.
+    int a_count = decoded.range.a_count();
+    unsigned valid = 0;
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i)
+      valid |= (unsigned)(nt * i + tid < a_count) << i;
+    typename tile_t::items_t x;
+    tiles.items(tid, decoded, shared, valid, x);
+
+    // All calls first, their results -- which usually come from memory --
+    // are only looked at afterwards, so the loads of all calls overlap.
+    int created[vt];
+    PRAGMA_UNROLL
+    for(int i = 0; i < vt; ++i) {
+      created[i] = 0;
+      if(valid & (1u << i))
+        created[i] = f(decoded.range.a_begin + nt * i + tid, x.seg[i],
+          x.rank[i], x.cached[i]);
+    }
     unsigned bits = 0;
     int work = 0;
     PRAGMA_UNROLL
     for(int i = 0; i < vt; ++i) {
-      if(nt * i + tid < decoded.range.a_count()) {
-        tiles.item(i, tid, decoded, shared,
-          [&](int index, int seg, int rank, value_t cached) {
-            int created = f(index, seg, rank, cached);
-            if(created > 0) {
-              bits |= 1u << i;
-              work += created;
-            }
-          });
+      if(created[i] > 0) {
+        bits |= 1u << i;
+        work += created[i];
       }
     }
     bits_data[nt * tile + tid] = bits;
@@ -200,12 +257,15 @@ struct workcreate_downsweep_f {
     int tile = xcd_tile(cta, tiles.num_tiles);
     if(tile >= tiles.num_tiles) return;
     __shared__ typename tile_t::storage_t shared;
+    // Tile positions of the creating items, in item order.
+    __shared__ typename tile_t::target_t targets[nt * vt];
 
     int lane = tid % warp_size, wave = tid / warp_size;
     unsigned bits = bits_data[nt * tile + tid];
     tile_total_t offset = offsets_data[tile];
 
-    // Position of every creating item among the tile's creating items.
+    // Position of every creating item among the tile's creating items; the
+    // items are gathered in that order into targets.
     int below[vt];
     PRAGMA_UNROLL
     for(int i = 0; i < vt; ++i) {
@@ -214,48 +274,86 @@ struct workcreate_downsweep_f {
       if(!lane) shared.table[num_waves * i + wave] = popc(creators);
     }
     int num_creators = tiles.scan_table(tid, shared);
-    int dest[vt];
-    PRAGMA_UNROLL
-    for(int i = 0; i < vt; ++i)
-      dest[i] = total_creators(offset) + shared.table[num_waves * i + wave] +
-        below[i];
-
-    // Tiles without a creating item have nothing to decode.  (The branch is
+    // Tiles without a creating item have nothing to do.  (The branch is
     // uniform: every thread has the same num_creators.)
     if(!num_creators) return;
-    typename tile_t::decoded_t decoded = tiles.decode(tid, tile, shared);
-
-    int created[vt];
     PRAGMA_UNROLL
     for(int i = 0; i < vt; ++i) {
-      created[i] = 0;
-      if(bits & (1u << i)) {
-        tiles.item(i, tid, decoded, shared,
+      if(bits & (1u << i))
+        targets[shared.table[num_waves * i + wave] + below[i]] =
+          (typename tile_t::target_t)(nt * i + tid);
+    }
+    // (decode() has barriers of its own before anything reads the targets.)
+    typename tile_t::decoded_t decoded = tiles.decode(tid, tile, shared);
+
+    // Creating item nt * r + tid in round r: every lane of a round has work,
+    // and what the callback stores under dest_seg is contiguous across the
+    // CTA.  What the calls return is only looked at after the last call.
+    int rounds = div_up(num_creators, (int)nt);
+    int dest_base = total_creators(offset);
+    int created[vt];
+    PRAGMA_UNROLL
+    for(int r = 0; r < vt; ++r) {
+      created[r] = 0;
+      int j = nt * r + tid;
+      if(r < rounds && j < num_creators)
+        tiles.item(targets[j], decoded, shared,
           [&](int index, int seg, int rank, value_t cached) {
-            created[i] = max(0, (int)f(dest[i], index, seg, rank, cached,
-              args...));
+            created[r] = f(dest_base + j, index, seg, rank, cached, args...);
           });
-      }
     }
 
     // Start of every new segment: work-items created in front of it.
     int before[vt];
     PRAGMA_UNROLL
-    for(int i = 0; i < vt; ++i) {
-      int inclusive = wave_scan(created[i], plus_t<int>(), lane);
-      before[i] = inclusive - created[i];
-      if(warp_size - 1 == lane)
-        shared.table[num_waves * i + wave] = inclusive;
+    for(int r = 0; r < vt; ++r) {
+      if(r < rounds) {
+        created[r] = max(created[r], 0);
+        int inclusive = wave_scan(created[r], plus_t<int>(), lane);
+        before[r] = inclusive - created[r];
+        if(warp_size - 1 == lane)
+          shared.table[num_waves * r + wave] = inclusive;
+      } else if(warp_size - 1 == lane)
+        shared.table[num_waves * r + wave] = 0;
     }
     tiles.scan_table(tid, shared);
     PRAGMA_UNROLL
-    for(int i = 0; i < vt; ++i) {
-      if(bits & (1u << i))
-        segments_output[dest[i]] = total_work(offset) +
-          shared.table[num_waves * i + wave] + before[i];
+    for(int r = 0; r < vt; ++r) {
+      int j = nt * r + tid;
+      if(r < rounds && j < num_creators)
+        segments_output[dest_base + j] = total_work(offset) +
+          shared.table[num_waves * r + wave] + before[r];
     }
   }
 };
+
+// The two kernels over caller-provided arrays: pairs = splits from
+// lbs_partition_tiles, bits = nt words per tile, totals / offsets = one
+// tile_total_t per tile (offsets is the exclusive scan of totals).
+template<typename launch_t, typename func_t, typename segments_it,
+  typename pointers_t>
+void workcreate_upsweep_launch(func_t f, pointers_t caching_iterators,
+  int count, segments_it segments, int num_segments, const int* pairs,
+  int num_tiles, unsigned* bits, tile_total_t* totals, context_t& context) {
+  typedef workcreate_tile_t<launch_t, segments_it, pointers_t> tile_t;
+  workcreate_upsweep_f<launch_t, func_t, segments_it, pointers_t> k {
+    tile_t { count, segments, num_segments, caching_iterators, pairs,
+      num_tiles }, f, bits, totals };
+  cta_launch<launch_t>(k, xcd_grid(num_tiles), context);
+}
+
+template<typename launch_t, typename func_t, typename segments_it,
+  typename pointers_t, typename... args_t>
+void workcreate_downsweep_launch(func_t f, pointers_t caching_iterators,
+  int count, segments_it segments, int num_segments, const int* pairs,
+  int num_tiles, const unsigned* bits, const tile_total_t* offsets,
+  int* segments_output, context_t& context, args_t... args) {
+  typedef workcreate_tile_t<launch_t, segments_it, pointers_t> tile_t;
+  workcreate_downsweep_f<launch_t, func_t, segments_it, pointers_t> k {
+    tile_t { count, segments, num_segments, caching_iterators, pairs,
+      num_tiles }, f, bits, offsets, segments_output };
+  cta_launch<launch_t>(k, xcd_grid(num_tiles), context, args...);
+}
 
 } // namespace detail
 
@@ -311,13 +409,10 @@ struct workcreate_t {
   count_t upsweep(func_t f, pointers_t caching_iterators) {
     if(!num_tiles) return count_t { 0, 0 };
 
-    typedef detail::workcreate_tile_t<launch_t, segments_it, pointers_t>
-      tile_t;
     mem_t<tile_total_t> totals(num_tiles, context);
-    detail::workcreate_upsweep_f<launch_t, func_t, segments_it, pointers_t>
-      k { tile_t { count, segments, num_segments, caching_iterators,
-        pairs.data(), num_tiles }, f, bits.data(), totals.data() };
-    cta_launch<launch_t>(k, mgpu::detail::xcd_grid(num_tiles), context);
+    detail::workcreate_upsweep_launch<launch_t>(f, caching_iterators, count,
+      segments, num_segments, pairs.data(), num_tiles, bits.data(),
+      totals.data(), context);
 
     // Offsets of every tile; the grand total goes to pinned host memory and
     // is there once the event has passed.
@@ -352,14 +447,9 @@ struct workcreate_t {
     mem_t<int> result(num_dest_segments, context);
     if(!num_tiles || !num_dest_segments) return result;
 
-    typedef detail::workcreate_tile_t<launch_t, segments_it, pointers_t>
-      tile_t;
-    detail::workcreate_downsweep_f<launch_t, func_t, segments_it, pointers_t>
-      k { tile_t { count, segments, num_segments, caching_iterators,
-        pairs.data(), num_tiles }, f, bits.data(), offsets.data(),
-        result.data() };
-    cta_launch<launch_t>(k, mgpu::detail::xcd_grid(num_tiles), context,
-      args...);
+    detail::workcreate_downsweep_launch<launch_t>(f, caching_iterators,
+      count, segments, num_segments, pairs.data(), num_tiles, bits.data(),
+      offsets.data(), result.data(), context, args...);
     return result;
   }
 

@@ -305,3 +305,34 @@ def reduce(values, op="plus", out=None, unsigned=False):
         _ptr(values), count, ctypes.c_void_p(out.data_ptr()), code, OPS[op],
         _ptr(ws), ws.numel(), _stream()))
     return out
+
+
+def workcreate(created, segments):
+    """Dynamic work creation (mgpu::expt::lbs_workcreate) with the per-item
+    counts in a tensor: item i of the workload described by ``segments``
+    creates a segment of ``created[i]`` new work-items, none if that is <= 0.
+
+    Returns ``(new_count, new_segments, source_index, source_seg,
+    source_rank)``: the number of work-items of the next pass, the start of
+    each new segment, and for each new segment the item that created it, that
+    item's segment and its rank there.  The sizes travel to the host between
+    the two sweeps, as in the reference's engine, so this call waits for the
+    stream once."""
+    _dev_i32(created, "created")
+    _dev_i32(segments, "segments")
+    count, num_segments = created.numel(), segments.numel()
+    need = lib().mgpu_hip_workcreate_workspace_bytes(count, num_segments)
+    ws = _workspace(need, created.device)
+    sizes = torch.zeros(2, dtype=torch.int32, device=created.device)
+    _check(lib().mgpu_hip_workcreate_upsweep(
+        _ptr(created), count, _ptr(segments), num_segments,
+        ctypes.c_void_p(sizes.data_ptr()), _ptr(ws), ws.numel(), _stream()))
+    num_new, new_count = (int(x) for x in sizes.tolist())
+    outs = [torch.empty(num_new, dtype=torch.int32, device=created.device)
+            for _ in range(4)]
+    if num_new:
+        _check(lib().mgpu_hip_workcreate_downsweep(
+            _ptr(created), count, _ptr(segments), num_segments,
+            _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(outs[3]),
+            _ptr(ws), ws.numel(), _stream()))
+    return (new_count,) + tuple(outs)

@@ -25,6 +25,10 @@
  *       oracle_transform_lbs on the tile's items; every tile item written by
  *       exactly one thread; popcount of a thread's low vt merge bits = items it
  *       takes; placements consecutive (a thread ends where the next begins).
+ *   oracle_workcreate : numpy flatnonzero / exclusive cumsum / searchsorted
+ *       closed forms; a breadth-first search that rebuilds its frontier with
+ *       it level by level (the loop of demo/bfs2.cu) against
+ *       scipy.sparse.csgraph shortest path lengths.
  *   oracle_interval_expand : numpy.repeat.
  *   oracle_spmv_* : scipy.sparse CSR product in float64.
  *   oracle_scan_* : numpy cumsum / maximum.accumulate / minimum.accumulate and
@@ -263,6 +267,40 @@ ORACLE_API void oracle_lbs_segreduce_seg_plus_rank(int count,
     }
     output[seg] = x;
   }
+}
+
+/* ------------------------------------------------------------------------- */
+/* expt::workcreate_t, kernel_workcreate.hxx:64-247, with the per-item count
+ * given as an array (the upsweep functor's return value for item `index`).
+ * Upsweep (:95-122): every item with a count > 0 creates one new segment
+ * (the bit test `work_count > 0`, :104) and the counts are summed.  Downsweep
+ * (:169-230): the creating items, in item order, are numbered dest_seg =
+ * 0, 1, ... (targets are compacted in thread order, which is item order, and
+ * tiles are offset by the scan of their counts, :203-204); the start of new
+ * segment dest_seg is the sum of the counts in front of it (:222-227); the
+ * functor sees (dest_seg, index, seg, rank) with seg and rank from the
+ * load-balancing search (:209-216).  The reference adds every count the
+ * functor returns to the total, positive or not; counts <= 0 are taken as 0
+ * here, which is the same for the non-negative counts it is meant for.
+ * Returns the number of new segments; *new_count = number of new work-items.
+ * Output arrays may be NULL (to size them first).                            */
+ORACLE_API int oracle_workcreate(const int* created, int count,
+  const int* segments, int num_segments, int* new_count, int* new_segments,
+  int* source_index, int* source_seg, int* source_rank) {
+  int dest_seg = 0, work = 0, seg = -1;
+  for(int index = 0; index < count; ++index) {
+    while(seg + 1 < num_segments && segments[seg + 1] <= index) ++seg;
+    if(created[index] > 0) {
+      if(new_segments) new_segments[dest_seg] = work;
+      if(source_index) source_index[dest_seg] = index;
+      if(source_seg) source_seg[dest_seg] = seg;
+      if(source_rank) source_rank[dest_seg] = index - (seg >= 0 ? segments[seg] : 0);
+      ++dest_seg;
+      work += created[index];
+    }
+  }
+  if(new_count) *new_count = work;
+  return dest_seg;
 }
 
 /* ------------------------------------------------------------------------- */

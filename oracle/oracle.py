@@ -198,6 +198,21 @@ def lbs_segreduce_seg_plus_rank(count, segments, init=-1):
     return out
 
 
+def workcreate(created, segments):
+    """(new_count, new_segments, source_index, source_seg, source_rank) of
+    expt::lbs_workcreate with the per-item counts in ``created``."""
+    c, s = _i32(created), _i32(segments)
+    fn = lib().oracle_workcreate
+    fn.restype = ctypes.c_int
+    new_count = ctypes.c_int(0)
+    n = fn(_p(c), int(c.size), _p(s), int(s.size), ctypes.byref(new_count),
+           None, None, None, None)
+    outs = [np.empty(n, dtype=np.int32) for _ in range(4)]
+    fn(_p(c), int(c.size), _p(s), int(s.size), ctypes.byref(new_count),
+       _p(outs[0]), _p(outs[1]), _p(outs[2]), _p(outs[3]))
+    return (new_count.value,) + tuple(outs)
+
+
 def cta_load_balance(count, segments, nt, vt, cta):
     """One tile of cta_load_balance_t::load_balance, thread by thread."""
     s = _i32(segments)

@@ -76,6 +76,16 @@ def test_bad_arguments_are_rejected_without_a_gpu():
     assert L.mgpu_hip_interval_expand(vp, 3, 10, vp, 2, vp, vp, 1 << 20, None) == HIP_ERROR_INVALID_VALUE
     assert L.mgpu_hip_load_balance_partitions(10, vp, 2, 0, vp, None) == HIP_ERROR_INVALID_VALUE
     assert L.mgpu_hip_merge_path_partitions(None, 10, vp, 2, 8, 7, vp, None) == HIP_ERROR_INVALID_VALUE
+    # workcreate: misaligned sizes, null counts, short workspace, index overflow
+    buf = (ctypes.c_int * 4)()
+    al = ctypes.cast(buf, ctypes.c_void_p)
+    mis = ctypes.c_void_p(al.value + 4)
+    assert L.mgpu_hip_workcreate_upsweep(al, 10, al, 1, mis, al, 1 << 20, None) == HIP_ERROR_INVALID_VALUE
+    assert L.mgpu_hip_workcreate_upsweep(None, 10, al, 1, al, al, 1 << 20, None) == HIP_ERROR_INVALID_VALUE
+    assert L.mgpu_hip_workcreate_upsweep(al, 10, al, 1, al, al, 8, None) == HIP_ERROR_INVALID_VALUE
+    assert L.mgpu_hip_workcreate_downsweep(al, 10, al, 1, None, None, None, None, al, 1 << 20, None) == HIP_ERROR_INVALID_VALUE
+    assert L.mgpu_hip_workcreate_workspace_bytes(1 << 30, 1 << 30) == 0
+    assert 0 < L.mgpu_hip_workcreate_workspace_bytes(1000, 10) < L.mgpu_hip_workcreate_workspace_bytes(1 << 24, 1 << 20)
     assert b"invalid" in L.mgpu_hip_error_string(HIP_ERROR_INVALID_VALUE).lower()
 
 

@@ -1,6 +1,6 @@
 """Runs the C++ callers written against the mgpu:: template API (same shape as
 the reference's tests/test_segreduce.cu and tests/test_load_balance.cu, plus
-user functors, user types and custom launch boxes).  They are compiled in-tree
+user functors, user types, custom launch boxes and the work-creation engine).  They are compiled in-tree
 by tests/csrc/Makefile and exit non-zero on any mismatch."""
 import os
 import subprocess
@@ -41,3 +41,7 @@ def test_reference_style_scan_and_reduce(dev):
 
 def test_reference_style_lbs_segreduce(dev):
     assert "all passed" in _run("test_lbs_segreduce", 4_000_000, 50_000)
+
+
+def test_workcreate_engine_and_bfs(dev):
+    assert "all passed" in _run("test_workcreate", 200_000)

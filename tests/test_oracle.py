@@ -422,3 +422,78 @@ def test_cta_load_balance_hand_example(oracle):
     assert list(r["range"][:2]) == [5, 10]
     assert list(r["a_index"]) == [5, 7, 8, 10]
     assert list(r["b_index"]) == [2, 2, 3, 3]
+
+
+# --- work creation -------------------------------------------------------------
+
+def _workcreate_numpy(created, segments):
+    created = np.asarray(created, dtype=np.int64)
+    who = np.flatnonzero(created > 0)
+    counts = created[who]
+    starts = np.cumsum(counts) - counts
+    seg = np.searchsorted(np.asarray(segments), who, side="right") - 1
+    rank = who - np.asarray(segments, dtype=np.int64)[seg] if who.size else who
+    return int(counts.sum()), starts, who, seg, rank
+
+
+def test_workcreate_vs_numpy(oracle):
+    rng = np.random.default_rng(77)
+    for count, nseg, keep in [(0, 0, 0.5), (0, 4, 0.5), (1, 1, 1.0), (50, 7, 0.5),
+                              (5000, 300, 0.1), (5000, 4000, 0.9), (3000, 1, 0.0)]:
+        segments = _random_segments(rng, count, nseg) if nseg else np.zeros(0, np.int32)
+        created = rng.integers(1, 9, size=count).astype(np.int32)
+        created[rng.random(count) >= keep] = 0
+        created[rng.random(count) < 0.05] = -3        # creates nothing either
+        got = oracle.workcreate(created, segments)
+        want = _workcreate_numpy(created, segments)
+        assert got[0] == want[0]
+        for g, w in zip(got[1:], want[1:]):
+            assert np.array_equal(g, w)
+
+
+def test_workcreate_hand_example(oracle):
+    # segments [0,3) [3,3) [3,7) [7,10); items 1, 3, 4 and 9 create 2, 1, 5, 4.
+    created = [0, 2, 0, 1, 5, 0, 0, 0, 0, 4]
+    got = oracle.workcreate(created, [0, 3, 3, 7])
+    assert got[0] == 12
+    assert got[1].tolist() == [0, 2, 3, 8]        # starts of the new segments
+    assert got[2].tolist() == [1, 3, 4, 9]        # creating items
+    assert got[3].tolist() == [0, 2, 2, 3]        # their segments
+    assert got[4].tolist() == [1, 0, 1, 2]        # their ranks
+
+
+def test_workcreate_bfs_vs_scipy(oracle):
+    """The frontier loop of the reference's demo/bfs2.cu with the oracle as the
+    engine: levels must be scipy's unweighted shortest path lengths."""
+    import scipy.sparse as sp
+    from scipy.sparse.csgraph import shortest_path
+    rng = np.random.default_rng(5)
+    n = 600
+    rows = np.concatenate([np.arange(n - 60), rng.integers(0, n - 60, 500)])
+    cols = np.concatenate([(np.arange(n - 60) + 1) % (n - 60), rng.integers(0, n - 60, 500)])
+    a = sp.coo_matrix((np.ones(rows.size), (rows, cols)), shape=(n, n))
+    a = ((a + a.T) > 0).astype(np.int8).tocsr()
+    indptr, indices = a.indptr.astype(np.int32), a.indices.astype(np.int32)
+    source = 23
+    want = shortest_path(a, unweighted=True, indices=source)
+    want = np.where(np.isinf(want), -1, want).astype(np.int32)
+
+    level = np.full(n, -1, dtype=np.int32)
+    level[source] = 0
+    segments = np.zeros(1, dtype=np.int32)
+    first_edge = np.array([indptr[source]], dtype=np.int32)
+    count, depth = int(indptr[source + 1] - indptr[source]), 0
+    while segments.size:
+        seg, rank = oracle.transform_lbs(count, segments)
+        created = np.zeros(count, dtype=np.int32)
+        for i in range(count):                      # the upsweep functor
+            w = indices[first_edge[seg[i]] + rank[i]]
+            if level[w] == -1:
+                level[w] = depth + 1
+                created[i] = indptr[w + 1] - indptr[w]
+        new_count, new_segments, src, src_seg, src_rank = oracle.workcreate(created, segments)
+        w = indices[first_edge[src_seg] + src_rank]  # the downsweep functor
+        assert np.array_equal(indptr[w + 1] - indptr[w], created[src])
+        segments, first_edge, count = new_segments, indptr[w], new_count
+        depth += 1
+    assert np.array_equal(level, want)
