@@ -222,6 +222,22 @@ MGPU_DEVICE inline void store_consecutive(type_t* dest,
   }
 }
 
+// The loading counterpart: W consecutive elements of any trivially copyable
+// type from an element-aligned address.
+template<int W, typename type_t>
+MGPU_DEVICE inline void load_consecutive(const type_t* source,
+  type_t (&x)[W]) {
+  if constexpr(0 == sizeof(type_t) % 4 && W * sizeof(type_t) <= 64) {
+    enum { words = W * sizeof(type_t) / 4 };
+    typedef unsigned v_t __attribute__((ext_vector_type(words), aligned(4)));
+    v_t v = *(const v_t*)source;
+    __builtin_memcpy(x, &v, sizeof(v));
+  } else {
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) x[e] = source[e];
+  }
+}
+
 } // namespace detail
 
 ////////////////////////////////////////////////////////////////////////////////

@@ -53,6 +53,66 @@ struct interval_copy_f {
   }
 };
 
+// Pointer to pointer: W consecutive items per call.  All W loads are issued
+// before the first store, and the side that is not gathered or scattered
+// moves as one 16-byte (or wider) access.
+template<bool scatters, bool gathers, typename type_t>
+struct interval_copy_chunks_f {
+  typedef void chunk_functor_tag;
+  const type_t* input;
+  type_t* output;
+
+  template<typename bases_t>
+  MGPU_DEVICE void operator()(int index, int, int rank, bases_t bases) const {
+    int from = index, to = index;
+    if constexpr(scatters) to = get<0>(bases) + rank;
+    if constexpr(gathers) from = get<scatters ? 1 : 0>(bases) + rank;
+    output[to] = input[from];
+  }
+
+  // Gathered elements are loaded one by one (W independent loads; measured
+  // faster than testing for a chunk that lies in one segment).  Scattered
+  // elements of one segment are consecutive and go out as one store -- W
+  // single stores per lane would each write a quarter of every cache line
+  // they touch -- and element by element when the chunk crosses a segment
+  // boundary.
+  template<int W, typename bases_t>
+  MGPU_DEVICE void chunk(int index, const int (&seg)[W], const int (&rank)[W],
+    const bases_t (&bases)[W]) const {
+    bool one_segment = seg[0] == seg[W - 1];
+    type_t x[W];
+    if constexpr(gathers) {
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e)
+        x[e] = input[get<scatters ? 1 : 0>(bases[e]) + rank[e]];
+    } else
+      load_consecutive<W>(input + index, x);
+    if constexpr(scatters) {
+      if(one_segment)
+        store_consecutive<W>(output + get<0>(bases[0]) + rank[0], x);
+      else {
+        PRAGMA_UNROLL
+        for(int e = 0; e < W; ++e) output[get<0>(bases[e]) + rank[e]] = x[e];
+      }
+    } else
+      store_consecutive<W>(output + index, x);
+  }
+};
+
+// The functor for a pair of iterator types.
+template<bool scatters, bool gathers, typename input_it, typename output_it>
+struct interval_copy_select_t {
+  typedef interval_copy_f<scatters, gathers, input_it, output_it> type;
+};
+template<bool scatters, bool gathers, typename type_t>
+struct interval_copy_select_t<scatters, gathers, const type_t*, type_t*> {
+  typedef interval_copy_chunks_f<scatters, gathers, type_t> type;
+};
+template<bool scatters, bool gathers, typename type_t>
+struct interval_copy_select_t<scatters, gathers, type_t*, type_t*> {
+  typedef interval_copy_chunks_f<scatters, gathers, type_t> type;
+};
+
 } // namespace detail
 
 // Segment s's one value written to each of its items:
@@ -73,8 +133,8 @@ template<typename launch_arg_t = empty_t, typename input_it,
   typename segments_it, typename gather_it, typename output_it>
 void interval_gather(input_it input, int count, segments_it segments,
   int num_segments, gather_it gather, output_it output, context_t& context) {
-  detail::interval_copy_f<false, true, input_it, output_it> copy {
-    input, output };
+  typename detail::interval_copy_select_t<false, true, input_it,
+    output_it>::type copy { input, output };
   transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
     make_tuple(gather), context);
 }
@@ -86,8 +146,8 @@ template<typename launch_arg_t = empty_t, typename input_it,
 void interval_scatter(input_it input, int count, segments_it segments,
   int num_segments, scatter_it scatter, output_it output,
   context_t& context) {
-  detail::interval_copy_f<true, false, input_it, output_it> copy {
-    input, output };
+  typename detail::interval_copy_select_t<true, false, input_it,
+    output_it>::type copy { input, output };
   transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
     make_tuple(scatter), context);
 }
@@ -99,8 +159,8 @@ template<typename launch_arg_t = empty_t,
 void interval_move(input_it input, int count, segments_it segments,
   int num_segments, scatter_it scatter, gather_it gather, output_it output,
   context_t& context) {
-  detail::interval_copy_f<true, true, input_it, output_it> copy {
-    input, output };
+  typename detail::interval_copy_select_t<true, true, input_it,
+    output_it>::type copy { input, output };
   transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
     make_tuple(scatter, gather), context);
 }

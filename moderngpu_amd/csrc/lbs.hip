@@ -43,30 +43,14 @@ typedef detail::lbs_store_seg_f<int*> store_seg_f;
 
 template<typename type_t>
 using expand_f = detail::interval_expand_f<type_t, type_t*>;
+// gather / scatter / move: the library's own pointer functors (W consecutive
+// items per call).
 template<typename type_t>
-struct gather_f {
-  const type_t* input; type_t* output;
-  MGPU_DEVICE void operator()(int index, int, int rank,
-    tuple<int> desc) const {
-    output[index] = input[get<0>(desc) + rank];
-  }
-};
+using gather_f = detail::interval_copy_chunks_f<false, true, type_t>;
 template<typename type_t>
-struct scatter_f {
-  const type_t* input; type_t* output;
-  MGPU_DEVICE void operator()(int index, int, int rank,
-    tuple<int> desc) const {
-    output[get<0>(desc) + rank] = input[index];
-  }
-};
+using scatter_f = detail::interval_copy_chunks_f<true, false, type_t>;
 template<typename type_t>
-struct move_f {
-  const type_t* input; type_t* output;
-  MGPU_DEVICE void operator()(int, int, int rank,
-    tuple<int, int> desc) const {
-    output[get<0>(desc) + rank] = input[get<1>(desc) + rank];
-  }
-};
+using move_f = detail::interval_copy_chunks_f<true, true, type_t>;
 
 template<int bytes>
 int expand_sized(const void* input, int count, const int* segments,
