@@ -506,11 +506,26 @@ struct cached_segment_load_t {
   // `count` must be the same in every thread.
   MGPU_DEVICE static bool stage(int tid, int begin, int count,
     storage_t& storage, pointers_t iterators) {
+    value_t x;
+    bool fits = fetch(tid, begin, count, iterators, x);
+    commit(tid, begin, count, x, storage);
+    return fits;
+  }
+  // The same in two steps, so that the global read can be in flight while
+  // the caller does something else (decodes the tile, say): fetch() issues
+  // the read into a register, commit() puts it into LDS and ends with a
+  // barrier if the values fit.
+  MGPU_DEVICE static bool fetch(int tid, int begin, int count,
+    pointers_t iterators, value_t& x) {
     if(count > nt) return false;
-    if(tid < count && begin + tid >= 0)
-      storage.data[tid] = mgpu::load(iterators, begin + tid);
-    __syncthreads();
+    if(tid < count && begin + tid >= 0) x = mgpu::load(iterators, begin + tid);
     return true;
+  }
+  MGPU_DEVICE static void commit(int tid, int begin, int count,
+    const value_t& x, storage_t& storage) {
+    if(count > nt) return;
+    if(tid < count && begin + tid >= 0) storage.data[tid] = x;
+    __syncthreads();
   }
   // Value of segment seg = begin + rel.
   MGPU_DEVICE static value_t get(bool staged, int rel, int seg,
@@ -549,6 +564,11 @@ struct cached_segment_load_t<nt, tuple<> > {
 
   MGPU_DEVICE static bool stage(int, int, int, storage_t&, tuple<>) {
     return false;
+  }
+  MGPU_DEVICE static bool fetch(int, int, int, tuple<>, value_t&) {
+    return false;
+  }
+  MGPU_DEVICE static void commit(int, int, int, const value_t&, storage_t&) {
   }
   MGPU_DEVICE static value_t get(bool, int, int, const storage_t&, tuple<>) {
     return value_t();

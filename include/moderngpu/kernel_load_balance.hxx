@@ -68,16 +68,20 @@ struct transform_lbs_f {
     // the tile's segment starts sit behind the slots.
     merge_range_t range = paired_tile_range(count, num_segments, tile,
       load_balance_t::nv, mp_data);
-    load_balance_t().fill(range, segments, tid, shared.lbs);
     int a_count = range.a_count();
     int seg_base = range.b_begin - 1;
+
+    // Items of the tile belong to segments [seg_base, b_end): their cached
+    // values are read once and fanned out through LDS when they fit.  The
+    // read is issued before the tile is decoded and lands while that runs.
+    value_t fetched;
+    bool staged = cached_load_t::fetch(tid, seg_base, range.b_count() + 1,
+      caching_iterators, fetched);
+    load_balance_t().fill(range, segments, tid, shared.lbs);
+    cached_load_t::commit(tid, seg_base, range.b_count() + 1, fetched,
+      shared.cached);
     const int* slots = shared.lbs.indices;
     const int* starts = slots + load_balance_t::starts_offset(a_count);
-
-    // Items of the tile belong to segments [seg_base, b_end): fetch their
-    // cached values once into LDS when they fit.
-    bool staged = cached_load_t::stage(tid, seg_base, range.b_count() + 1,
-      shared.cached, caching_iterators);
 
     // The emission loop exists twice -- cached values staged in LDS, or
     // gathered from global memory -- so that each copy is straight-line code.

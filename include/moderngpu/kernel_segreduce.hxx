@@ -313,11 +313,15 @@ struct segreduce_tile_f {
       typedef cached_segment_load_t<nt, pointers_t> cached_load_t;
       int a_count = range.a_count();
       int seg_base = range.b_begin - 1;
+      // The cached values' read is in flight while the tile is decoded.
+      typename cached_load_t::value_t fetched;
+      bool staged = cached_load_t::fetch(tid, seg_base, range.b_count() + 1,
+        input.caching_iterators, fetched);
       load_balance_t().fill(range, segments, tid, shared.source.lbs);
+      cached_load_t::commit(tid, seg_base, range.b_count() + 1, fetched,
+        shared.source.cached);
       const int* slots = shared.source.lbs.indices;
       const int* starts = slots + load_balance_t::starts_offset(a_count);
-      bool staged = cached_load_t::stage(tid, seg_base, range.b_count() + 1,
-        shared.source.cached, input.caching_iterators);
       PRAGMA_UNROLL
       for(int i = 0; i < chunks; ++i) {
         PRAGMA_UNROLL

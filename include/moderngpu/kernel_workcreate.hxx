@@ -107,9 +107,13 @@ struct workcreate_tile_t {
   MGPU_DEVICE decoded_t decode(int tid, int tile, storage_t& shared) const {
     merge_range_t range = paired_tile_range(count, num_segments, tile,
       load_balance_t::nv, pairs);
+    // The cached values' read is in flight while the tile is decoded.
+    value_t fetched;
+    bool staged = cached_load_t::fetch(tid, range.b_begin - 1,
+      range.b_count() + 1, caching_iterators, fetched);
     load_balance_t().fill(range, segments, tid, shared.lbs);
-    bool staged = cached_load_t::stage(tid, range.b_begin - 1,
-      range.b_count() + 1, shared.cached, caching_iterators);
+    cached_load_t::commit(tid, range.b_begin - 1, range.b_count() + 1,
+      fetched, shared.cached);
     return decoded_t { range, staged };
   }
 
