@@ -141,6 +141,83 @@ def make_c3(copies, expand=False):
     return wk
 
 
+def make_c3_moves(copies, kind):
+    """interval_gather / interval_scatter / interval_move on the C3 segments:
+    every segment's items live, on the gathered or scattered side, at a
+    random place of their own (the segments laid out in a random order)."""
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    from oracle import oracle
+    copies = min(copies, 2)
+    w = workloads.config3()
+    n, s = w["count"], w["segments"].size
+    lengths = np.diff(np.append(w["segments"].astype(np.int64), n))
+    order = np.random.Generator(np.random.PCG64(43)).permutation(s)
+    base = np.zeros(s, dtype=np.int64)
+    base[order] = np.cumsum(lengths[order]) - lengths[order]
+    base = base.astype(np.int32)
+    segs = [_dev(w["segments"]) for _ in range(copies)]
+    bases = [_dev(base) for _ in range(copies)]
+    inp_host = np.random.Generator(np.random.PCG64(44)).integers(
+        0, 2 ** 31, size=n, dtype=np.int64).astype(np.int32)
+    inps = [_dev(inp_host) for _ in range(copies)]
+    outs = [torch.empty(n, dtype=torch.int32, device="cuda") for _ in range(copies)]
+    wk = Workload()
+    wk.dtype, wk.items = "i32", n
+    wk.key = "c3_interval_%s_i32" % kind
+    wk.name = "interval_%s int32, 2^24 Zipf(1.2) segments, 2^28 items, segments placed " \
+              "in random order" % kind
+    wk.kernel = "transform_lbs_f<512x12, %s> (whole call)" % kind
+    wk.bytes = n * 4 + n * 4 + s * 4 + s * 4 * (2 if kind == "move" else 1)
+    if kind == "gather":
+        wk.step = lambda i: m.interval_gather(inps[i % copies], n, segs[i % copies],
+                                              bases[i % copies], out=outs[i % copies])
+        want = lambda: oracle.interval_gather(inp_host, n, w["segments"], base)
+    elif kind == "scatter":
+        wk.step = lambda i: m.interval_scatter(inps[i % copies], n, segs[i % copies],
+                                               bases[i % copies], outs[i % copies])
+        want = lambda: oracle.interval_scatter(inp_host, n, w["segments"], base, n)
+    else:
+        # move = gather from the random layout back to segment order
+        wk.step = lambda i: m.interval_move(inps[i % copies], n, segs[i % copies],
+                                            segs[i % copies], bases[i % copies],
+                                            outs[i % copies])
+        want = lambda: oracle.interval_move(inp_host, n, w["segments"], w["segments"],
+                                            base, n)
+    wk.tiles = wk.step
+    wk.check = lambda: bool(np.array_equal(wk.step(0).cpu().numpy(), want()))
+    wk.cpu = lambda: want
+    return wk
+
+
+def make_lbs_segreduce(copies):
+    """lbs_segreduce with the reference test's functor (seg + rank) on the C2
+    segments: the items are computed, so the only traffic is the starts in
+    and one sum per segment out."""
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    from oracle import oracle
+    w = workloads.config2()
+    n, s = w["values"].size, w["segments"].size
+    segs = [_dev(w["segments"]) for _ in range(copies)]
+    outs = [torch.empty(s, dtype=torch.int32, device="cuda") for _ in range(copies)]
+    wk = Workload()
+    wk.dtype, wk.items = "i32", n
+    wk.key = "c2_lbs_segreduce_i32"
+    wk.name = "lbs_segreduce f = seg + rank, int32 plus, 2^26 computed items, 2^20 segments"
+    wk.kernel = "segreduce_tile_f<lbs input> + partition + spine (whole call)"
+    wk.bytes = s * 4 + s * 4
+    wk.step = lambda i: m.lbs_segreduce_seg_plus_rank(n, segs[i % copies], -1,
+                                                      out=outs[i % copies])
+    wk.tiles = wk.step
+    wk.check = lambda: bool(np.array_equal(
+        wk.step(0).cpu().numpy(), oracle.lbs_segreduce_seg_plus_rank(n, w["segments"], -1)))
+    wk.cpu = lambda: (lambda: oracle.lbs_segreduce_seg_plus_rank(n, w["segments"], -1))
+    return wk
+
+
 def make_c4(copies):
     import torch
     import moderngpu_amd as m
@@ -343,6 +420,10 @@ FACTORIES = {
     "c2_segreduce_f32": make_c2,
     "c3_load_balance_search": lambda c: make_c3(c, False),
     "c3_interval_expand_i32": lambda c: make_c3(c, True),
+    "c3_interval_gather_i32": lambda c: make_c3_moves(c, "gather"),
+    "c3_interval_scatter_i32": lambda c: make_c3_moves(c, "scatter"),
+    "c3_interval_move_i32": lambda c: make_c3_moves(c, "move"),
+    "c2_lbs_segreduce_i32": make_lbs_segreduce,
     "c4_spmv_f32": make_c4,
     "c5_f64max": lambda c: make_c5(c, "f64max"),
     "c5_i64sum": lambda c: make_c5(c, "i64sum"),
