@@ -103,12 +103,13 @@ MGPU_DEVICE inline merge_range_t tile_range(int count, int num_segments,
   int cta, int nv, int mp0, int mp1) {
   int total = count + num_segments;
   int diag0 = nv * cta;
-  int diag1 = min(total, diag0 + nv);
+  int diag1 = diag0 + min(nv, total - diag0);      // no overflow near 2^31
   mp0 = min(max(mp0, max(0, diag0 - num_segments)), min(diag0, count));
   mp1 = min(max(mp1, max(0, diag1 - num_segments)), min(diag1, count));
-  mp1 = min(max(mp1, mp0), mp0 + nv);
+  mp1 = mp0 + min(max(mp1 - mp0, 0), nv);
   merge_range_t r { mp0, mp1, diag0 - mp0, diag1 - mp1 };
-  r.b_end = min(max(r.b_end, r.b_begin), r.b_begin + nv - (mp1 - mp0));
+  r.b_end = r.b_begin +
+    min(max(r.b_end - r.b_begin, 0), nv - (mp1 - mp0));
   return r;
 }
 
@@ -140,8 +141,8 @@ MGPU_DEVICE inline merge_range_t paired_tile_range(int count,
   int a1 = pairs[2 * tile + 2], b1 = pairs[2 * tile + 3];
   a0 = min(max(a0, 0), count);
   b0 = min(max(b0, 0), num_segments);
-  a1 = min(min(max(a1, a0), a0 + nv), count);
-  b1 = min(min(max(b1, b0), b0 + nv - (a1 - a0)), num_segments);
+  a1 = min(a0 + min(max(a1 - a0, 0), nv), count);
+  b1 = min(b0 + min(max(b1 - b0, 0), nv - (a1 - a0)), num_segments);
   return merge_range_t { a0, a1, b0, b1 };
 }
 

@@ -60,7 +60,7 @@ MGPU_HOST_DEVICE bool merge_predicate(type_t a_key, type_t b_key,
 MGPU_HOST_DEVICE merge_range_t compute_merge_range(int a_count, int b_count,
   int partition, int spacing, int mp0, int mp1) {
   int diag0 = spacing * partition;
-  int diag1 = min(a_count + b_count, diag0 + spacing);
+  int diag1 = diag0 + min(spacing, a_count + b_count - diag0);
   return merge_range_t { mp0, mp1, diag0 - mp0, diag1 - mp1 };
 }
 

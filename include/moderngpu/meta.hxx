@@ -55,12 +55,16 @@ using enable_if_t = typename std::enable_if<condition, type_t>::type;
 
 // ceil(x / y) for non-negative x and positive y, in the three index widths
 // the library uses (plain overloads, so enumerators and mixed int arguments
-// convert).
+// convert).  The int form adds in unsigned arithmetic: x + y - 1 may pass
+// 2^31 for item counts close to the index limit.
+MGPU_HOST_DEVICE constexpr int div_up(int x, int y) {
+  return (int)(((unsigned)x + (unsigned)y - 1u) / (unsigned)y);
+}
 #define MGPU_DIV_UP(int_t)                                                    \
   MGPU_HOST_DEVICE constexpr int_t div_up(int_t x, int_t y) {                 \
     return (x + y - 1) / y;                                                   \
   }
-MGPU_DIV_UP(int) MGPU_DIV_UP(int64_t) MGPU_DIV_UP(size_t)
+MGPU_DIV_UP(int64_t) MGPU_DIV_UP(size_t)
 #undef MGPU_DIV_UP
 MGPU_HOST_DEVICE constexpr bool is_pow2(int x) { return !(x & (x - 1)); }
 

@@ -182,7 +182,8 @@ struct lbs_partition_scatter_f {
     int tile_at[vt + 1];
     PRAGMA_UNROLL
     for(int e = 0; e <= vt; ++e)
-      tile_at[e] = tile_of(min(max(starts[e] + j0 + e, 0), total));
+      tile_at[e] = tile_of(min(max(starts[e] + min(j0 + e, num_segments), 0),
+        total));
 
     // Few segments have a split behind them (one in spacing / mean segment
     // length), so everything but the test for it sits inside the branch.

@@ -64,8 +64,8 @@ struct MGPU_ALIGN(8) range_t {
 // Items [nv * cta, nv * (cta + 1)) of `count`, clipped at the end.
 MGPU_HOST_DEVICE range_t get_tile(int cta, int nv, int count) {
   int first = nv * cta;
-  int last = first + nv;
-  return range_t { first, last < count ? last : count };
+  int left = count - first;                 // first + nv may not fit an int
+  return range_t { first, first + (left < nv ? left : nv) };
 }
 
 // A tile of a two-input merge: items (A) and segment starts (B).
