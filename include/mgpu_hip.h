@@ -250,6 +250,45 @@ MGPU_HIP_API int mgpu_hip_workcreate_downsweep(const int* created, int count,
   int* source_index, int* source_seg, int* source_rank, void* workspace,
   size_t workspace_bytes, mgpu_stream_t stream);
 
+/* ---- sorted search and join (callers of the search) ---------------------- */
+
+/* Bytes of workspace mgpu_hip_sorted_search needs (the tile splits). */
+MGPU_HIP_API size_t mgpu_hip_sorted_search_workspace_bytes(int num_needles,
+  int num_haystack);
+
+/* mgpu::sorted_search<bounds> (kernel_sortedsearch.hxx:7-73) for int keys
+ * ordered by less_t; both arrays ascending.  indices[i] = number of haystack
+ * keys less than needles[i] (MGPU_BOUNDS_LOWER) or not greater than it
+ * (MGPU_BOUNDS_UPPER). */
+MGPU_HIP_API int mgpu_hip_sorted_search(const int* needles, int num_needles,
+  const int* haystack, int num_haystack, int bounds, int* indices,
+  void* workspace, size_t workspace_bytes, mgpu_stream_t stream);
+
+/* mgpu::inner_join (kernel_join.hxx:9-51) for ascending int keys, in the two
+ * steps its data-dependent output size forces (the reference reads the count
+ * back and allocates in between, :33-36).
+ *
+ * Step 1 (sorted searches + scan of the match counts, :14-31): stores the
+ * number of pairs to *join_count (device memory, or host memory the device
+ * can write) and leaves what step 2 needs in `workspace`
+ * (mgpu_hip_inner_join_workspace_bytes(a_count, b_count) bytes). */
+MGPU_HIP_API size_t mgpu_hip_inner_join_workspace_bytes(int a_count,
+  int b_count);
+MGPU_HIP_API int mgpu_hip_inner_join_count(const int* a, int a_count,
+  const int* b, int b_count, int* join_count, void* workspace,
+  size_t workspace_bytes, mgpu_stream_t stream);
+
+/* Step 2 (the load-balancing search, :38-46): pairs[2 * k] = index into a,
+ * pairs[2 * k + 1] = index into b of the k-th pair, ordered by a index, then
+ * b index; pairs is 8-byte aligned.  count_workspace is step 1's workspace,
+ * untouched since; workspace is a second one of
+ * mgpu_hip_inner_join_pairs_workspace_bytes(a_count, join_count) bytes. */
+MGPU_HIP_API size_t mgpu_hip_inner_join_pairs_workspace_bytes(int a_count,
+  int64_t join_count);
+MGPU_HIP_API int mgpu_hip_inner_join_pairs(int a_count, int b_count,
+  int join_count, const void* count_workspace, int* pairs, void* workspace,
+  size_t workspace_bytes, mgpu_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -38,6 +38,12 @@ SIGNATURES = {
     "mgpu_hip_scan": (c_int, [c_vp, c_int, c_vp, c_int, c_int, c_int, c_vp, c_vp, c_size, c_vp]),
     "mgpu_hip_reduce_workspace_bytes": (c_size, [c_int, c_int]),
     "mgpu_hip_reduce": (c_int, [c_vp, c_int, c_vp, c_int, c_int, c_vp, c_size, c_vp]),
+    "mgpu_hip_sorted_search_workspace_bytes": (c_size, [c_int, c_int]),
+    "mgpu_hip_sorted_search": (c_int, [c_vp, c_int, c_vp, c_int, c_int, c_vp, c_vp, c_size, c_vp]),
+    "mgpu_hip_inner_join_workspace_bytes": (c_size, [c_int, c_int]),
+    "mgpu_hip_inner_join_count": (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_size, c_vp]),
+    "mgpu_hip_inner_join_pairs_workspace_bytes": (c_size, [c_int, c_i64]),
+    "mgpu_hip_inner_join_pairs": (c_int, [c_int, c_int, c_int, c_vp, c_vp, c_vp, c_size, c_vp]),
     "mgpu_hip_workcreate_workspace_bytes": (c_size, [c_int, c_int]),
     "mgpu_hip_workcreate_upsweep": (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_size, c_vp]),
     "mgpu_hip_workcreate_downsweep": (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_vp, c_vp, c_vp, c_vp, c_size, c_vp]),

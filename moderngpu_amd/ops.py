@@ -336,3 +336,44 @@ def workcreate(created, segments):
             _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(outs[3]),
             _ptr(ws), ws.numel(), _stream()))
     return (new_count,) + tuple(outs)
+
+
+def sorted_search(needles, haystack, bounds="lower", out=None):
+    """out[i] = lower or upper bound of needles[i] in haystack
+    (mgpu::sorted_search); both int32 and ascending."""
+    _dev_i32(needles, "needles")
+    _dev_i32(haystack, "haystack")
+    n, h = needles.numel(), haystack.numel()
+    if out is None:
+        out = torch.empty(n, dtype=torch.int32, device=needles.device)
+    ws = _workspace(lib().mgpu_hip_sorted_search_workspace_bytes(n, h), needles.device)
+    _check(lib().mgpu_hip_sorted_search(
+        _ptr(needles), n, _ptr(haystack), h, {"lower": 0, "upper": 1}[bounds],
+        _ptr(out), _ptr(ws), ws.numel(), _stream()))
+    return out
+
+
+def inner_join(a, b):
+    """All pairs (i, j) with a[i] == b[j] for ascending int32 keys
+    (mgpu::inner_join), as an (n, 2) int32 tensor ordered by i, then j.  The
+    number of pairs travels to the host between the two steps, as in the
+    reference, so this call waits for the stream once."""
+    _dev_i32(a, "a")
+    _dev_i32(b, "b")
+    na, nb = a.numel(), b.numel()
+    need = lib().mgpu_hip_inner_join_workspace_bytes(na, nb)
+    ws1 = torch.empty(max(int(need), 256), dtype=torch.uint8, device=a.device)
+    count = torch.zeros(1, dtype=torch.int32, device=a.device)
+    _check(lib().mgpu_hip_inner_join_count(
+        _ptr(a), na, _ptr(b), nb, ctypes.c_void_p(count.data_ptr()),
+        _ptr(ws1), ws1.numel(), _stream()))
+    n = int(count.item())
+    pairs = torch.empty((n, 2), dtype=torch.int32, device=a.device)
+    if n:
+        need = lib().mgpu_hip_inner_join_pairs_workspace_bytes(na, n)
+        if not need:
+            raise MgpuError(1)
+        ws2 = _workspace(need, a.device)
+        _check(lib().mgpu_hip_inner_join_pairs(
+            na, nb, n, _ptr(ws1), _ptr(pairs), _ptr(ws2), ws2.numel(), _stream()))
+    return pairs

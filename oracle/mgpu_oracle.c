@@ -29,6 +29,9 @@
  *       closed forms; a breadth-first search that rebuilds its frontier with
  *       it level by level (the loop of demo/bfs2.cu) against
  *       scipy.sparse.csgraph shortest path lengths.
+ *   oracle_sorted_search / oracle_inner_join : numpy.searchsorted (left /
+ *       right), the assertions of the reference's own test
+ *       (tests/test_sortedsearch.cu:24-25), brute force over all pairs.
  *   oracle_interval_expand : numpy.repeat.
  *   oracle_spmv_* : scipy.sparse CSR product in float64.
  *   oracle_scan_* : numpy cumsum / maximum.accumulate / minimum.accumulate and
@@ -301,6 +304,44 @@ ORACLE_API int oracle_workcreate(const int* created, int count,
   }
   if(new_count) *new_count = work;
   return dest_seg;
+}
+
+/* ------------------------------------------------------------------------- */
+/* sorted_search<bounds>, kernel_sortedsearch.hxx:7-73, int keys with less_t:
+ * the serial merge of the two sorted arrays that the kernel performs per
+ * thread (cta_merge.hxx serial_merge through merge_predicate, :41-49 here
+ * restated): with bounds_lower a needle is taken while !(hay < needle), i.e.
+ * in front of equal haystack keys; with bounds_upper while needle < hay fails
+ * to hold for the haystack key, i.e. behind them.  indices[i] = haystack keys
+ * consumed when needle i is taken (:52-57).                                  */
+ORACLE_API void oracle_sorted_search(const int* needles, int num_needles,
+  const int* haystack, int num_haystack, int upper, int* indices) {
+  int h = 0;
+  for(int i = 0; i < num_needles; ++i) {
+    int key = needles[i];
+    while(h < num_haystack &&
+      (upper ? !(key < haystack[h]) : (haystack[h] < key))) ++h;
+    indices[i] = h;
+  }
+}
+
+/* inner_join, kernel_join.hxx:9-51: for every a key its matches are
+ * b[lower, upper) (:14-20), the pairs are laid out by the scan of the match
+ * counts (:27-31) and pair number `rank` of key `seg` is
+ * (seg, lower[seg] + rank) (:41-43).  Returns the number of pairs; pairs may
+ * be NULL to count only.                                                     */
+ORACLE_API int64_t oracle_inner_join(const int* a, int a_count, const int* b,
+  int b_count, int* pairs) {
+  int64_t n = 0;
+  int lo = 0, hi = 0;
+  for(int i = 0; i < a_count; ++i) {
+    while(lo < b_count && b[lo] < a[i]) ++lo;
+    if(hi < lo) hi = lo;
+    while(hi < b_count && !(a[i] < b[hi])) ++hi;
+    for(int j = lo; j < hi; ++j, ++n)
+      if(pairs) { pairs[2 * n] = i; pairs[2 * n + 1] = j; }
+  }
+  return n;
 }
 
 /* ------------------------------------------------------------------------- */

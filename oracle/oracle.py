@@ -213,6 +213,25 @@ def workcreate(created, segments):
     return (new_count.value,) + tuple(outs)
 
 
+def sorted_search(needles, haystack, upper=False):
+    n, h = _i32(needles), _i32(haystack)
+    out = np.empty(n.size, dtype=np.int32)
+    lib().oracle_sorted_search(_p(n), int(n.size), _p(h), int(h.size), int(bool(upper)),
+                               _p(out))
+    return out
+
+
+def inner_join(a, b):
+    """(n, 2) int32 array of (a index, b index), ordered by a index then b."""
+    x, y = _i32(a), _i32(b)
+    fn = lib().oracle_inner_join
+    fn.restype = ctypes.c_int64
+    n = fn(_p(x), int(x.size), _p(y), int(y.size), None)
+    pairs = np.empty((n, 2), dtype=np.int32)
+    fn(_p(x), int(x.size), _p(y), int(y.size), _p(pairs))
+    return pairs
+
+
 def cta_load_balance(count, segments, nt, vt, cta):
     """One tile of cta_load_balance_t::load_balance, thread by thread."""
     s = _i32(segments)

@@ -45,3 +45,7 @@ def test_reference_style_lbs_segreduce(dev):
 
 def test_workcreate_engine_and_bfs(dev):
     assert "all passed" in _run("test_workcreate", 200_000)
+
+
+def test_reference_style_sorted_search_and_join(dev):
+    assert "all passed" in _run("test_join")

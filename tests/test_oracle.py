@@ -497,3 +497,33 @@ def test_workcreate_bfs_vs_scipy(oracle):
         segments, first_edge, count = new_segments, indptr[w], new_count
         depth += 1
     assert np.array_equal(level, want)
+
+
+# --- sorted search and join ------------------------------------------------------
+
+def test_sorted_search_vs_numpy_and_reference_test_assertions(oracle):
+    rng = np.random.default_rng(91)
+    for n, h, hi in [(0, 10, 5), (10, 0, 5), (1000, 1000, 10000), (5000, 300, 50),
+                     (300, 5000, 50), (2000, 2000, 3)]:
+        needles = np.sort(rng.integers(0, hi + 1, size=n)).astype(np.int32)
+        haystack = np.sort(rng.integers(0, hi + 1, size=h)).astype(np.int32)
+        lower = oracle.sorted_search(needles, haystack, upper=False)
+        upper = oracle.sorted_search(needles, haystack, upper=True)
+        assert np.array_equal(lower, np.searchsorted(haystack, needles, side="left"))
+        assert np.array_equal(upper, np.searchsorted(haystack, needles, side="right"))
+        # what tests/test_sortedsearch.cu asserts for bounds_lower
+        for i, index in enumerate(lower):
+            assert index <= 0 or needles[i] > haystack[index - 1]
+            assert index >= h or needles[i] <= haystack[index]
+
+
+def test_inner_join_vs_brute_force(oracle):
+    rng = np.random.default_rng(92)
+    for na, nb, hi in [(0, 0, 3), (0, 7, 3), (7, 0, 3), (60, 80, 10), (200, 150, 1000),
+                       (50, 50, 0)]:
+        a = np.sort(rng.integers(0, hi + 1, size=na)).astype(np.int32)
+        b = np.sort(rng.integers(0, hi + 1, size=nb)).astype(np.int32)
+        want = [(i, j) for i in range(na) for j in range(nb) if a[i] == b[j]]
+        got = oracle.inner_join(a, b)
+        assert got.shape == (len(want), 2)
+        assert [tuple(p) for p in got.tolist()] == want
