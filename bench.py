@@ -218,6 +218,51 @@ def make_lbs_segreduce(copies):
     return wk
 
 
+def make_search(copies, kind):
+    """sorted_search: 2^26 sorted needles in 2^26 sorted haystack keys, both
+    uniform in [0, 2^28).  inner_join: 2^24 keys a side, uniform in [0, 2^24)
+    (about one match per key)."""
+    import torch
+    import moderngpu_amd as m
+    from oracle import oracle
+    rng = np.random.Generator(np.random.PCG64(42))
+    wk = Workload()
+    wk.dtype = "i32"
+    if kind == "search":
+        n = h = 1 << 26
+        needles = np.sort(rng.integers(0, 1 << 28, size=n, dtype=np.int32))
+        haystack = np.sort(rng.integers(0, 1 << 28, size=h, dtype=np.int32))
+        dn = [_dev(needles) for _ in range(copies)]
+        dh = [_dev(haystack) for _ in range(copies)]
+        outs = [torch.empty(n, dtype=torch.int32, device="cuda") for _ in range(copies)]
+        wk.key, wk.items = "sorted_search_i32", n
+        wk.name = "sorted_search lower bound, 2^26 needles in 2^26 haystack keys"
+        wk.bytes = n * 4 + h * 4 + n * 4
+        wk.kernel = "merge_path_partition_f + sorted_search_f<256x12> (whole call)"
+        wk.step = lambda i: m.sorted_search(dn[i % copies], dh[i % copies], "lower",
+                                            out=outs[i % copies])
+        wk.check = lambda: bool(np.array_equal(
+            wk.step(0).cpu().numpy(), np.searchsorted(haystack, needles, side="left")))
+        wk.cpu = lambda: (lambda: oracle.sorted_search(needles, haystack))
+    else:
+        n = 1 << 24
+        a = np.sort(rng.integers(0, n, size=n, dtype=np.int32))
+        b = np.sort(rng.integers(0, n, size=n, dtype=np.int32))
+        da = [_dev(a) for _ in range(copies)]
+        db = [_dev(b) for _ in range(copies)]
+        pairs = int(oracle.inner_join(a, b).shape[0])
+        wk.key, wk.items = "inner_join_i32", 2 * n
+        wk.name = "inner_join, 2^24 keys a side, %d pairs" % pairs
+        wk.bytes = 2 * n * 4 + pairs * 8
+        wk.kernel = "2 x sorted_search + scan + transform_lbs (whole call, one host wait)"
+        wk.step = lambda i: m.inner_join(da[i % copies], db[i % copies])
+        wk.check = lambda: bool(np.array_equal(wk.step(0).cpu().numpy(),
+                                               oracle.inner_join(a, b)))
+        wk.cpu = lambda: (lambda: oracle.inner_join(a, b))
+    wk.tiles = wk.step
+    return wk
+
+
 def make_c4(copies):
     import torch
     import moderngpu_amd as m
@@ -424,6 +469,8 @@ FACTORIES = {
     "c3_interval_scatter_i32": lambda c: make_c3_moves(c, "scatter"),
     "c3_interval_move_i32": lambda c: make_c3_moves(c, "move"),
     "c2_lbs_segreduce_i32": make_lbs_segreduce,
+    "sorted_search_i32": lambda c: make_search(c, "search"),
+    "inner_join_i32": lambda c: make_search(c, "join"),
     "c4_spmv_f32": make_c4,
     "c5_f64max": lambda c: make_c5(c, "f64max"),
     "c5_i64sum": lambda c: make_c5(c, "i64sum"),
