@@ -193,7 +193,7 @@ struct pointer_loader_t {
     const type_t* tile = input + base;
     if constexpr(W > 1) {
       typedef typename vec_t<type_t, W>::type_u v_t;
-      v_t v = *(const v_t*)(tile + offset);
+      v_t v = __builtin_nontemporal_load((const v_t*)(tile + offset));
       PRAGMA_UNROLL
       for(int e = 0; e < W; ++e) x[e] = v[e];
     } else
