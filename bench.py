@@ -480,11 +480,11 @@ FACTORIES = {
 # FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by what the same counters
 # read for a plain copy of known size.  None until measured.
 TRAFFIC_BYTES = {
-    # profiles/segreduce_tile_f__c2_segreduce_f32.md: FETCH 133,785.8 KiB x 2.000
-    # + WRITE 4,286.2 KiB x 1.000
-    "c2_segreduce_f32": int((133785.8 * 2.000 + 4286.2) * 1024),
+    # profiles/segreduce_tile_f__c2_segreduce_f32.md: FETCH 134,994.4 KiB x 2.000
+    # + WRITE 4,255.6 KiB x 1.000
+    "c2_segreduce_f32": int((134994.4 * 2.000 + 4255.6) * 1024),
     # profiles/transform_lbs_f__c3_load_balance_search.md
-    "c3_load_balance_search": int((33529.9 * 2.000 + 1048576.1) * 1024),
+    "c3_load_balance_search": int((33532.2 * 2.000 + 1048576.1) * 1024),
 }
 
 

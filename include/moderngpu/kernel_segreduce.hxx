@@ -172,9 +172,10 @@ struct segscan_thread_t<vt, vt> {
 };
 
 ////////////////////////////////////////////////////////////////////////////////
-// Default tiles on gfx950: 256 threads x 16 values for 4- and 8-byte values
-// (16 KB / 32 KB of values in LDS); wider value types get fewer values per
-// thread so that the tile stays under the 64 KB a workgroup may declare.
+// Default tiles on gfx950: 16 values per thread, 256 threads for 4-byte values
+// and 128 for 8-byte ones (16 KB of values in LDS either way); wider value
+// types get fewer values per thread so that the tile stays under the 64 KB a
+// workgroup may declare.
 
 template<typename type_t>
 struct segreduce_launch_default_t {
@@ -182,7 +183,9 @@ struct segreduce_launch_default_t {
     vt = sizeof(type_t) <= 8 ? 16 :
       (128 / sizeof(type_t) > 1 ? 128 / sizeof(type_t) : 1)
   };
-  typedef launch_box_t<arch_gfx950_cta<256, vt> > type_t_;
+  // 8-byte values: half the threads for the same bytes per tile.
+  typedef launch_box_t<arch_gfx950_cta<(sizeof(type_t) == 8 ? 128 : 256),
+    vt> > type_t_;
 };
 
 ////////////////////////////////////////////////////////////////////////////////
