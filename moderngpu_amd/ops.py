@@ -103,6 +103,49 @@ def segreduce(values, segments, op="plus", init=0, out=None, unsigned=False,
     return out
 
 
+def prepare_segreduce(values, segments, op="plus", init=0, out=None, unsigned=False,
+                      phases=7):
+    """segreduce() for a caller that repeats one call: arguments are checked
+    and converted once, and the returned zero-argument callable only makes the
+    C call (on the stream that is current now).  Returns (callable, out)."""
+    _dev_i32(segments, "segments")
+    if not values.is_cuda or not values.is_contiguous():
+        raise TypeError("values must be a contiguous CUDA tensor")
+    code = _dtype_code(values, unsigned)
+    count, nseg = values.numel(), segments.numel()
+    if out is None:
+        out = torch.empty(nseg, dtype=values.dtype, device=values.device)
+    need = lib().mgpu_hip_segreduce_workspace_bytes(count, nseg, code)
+    ws = _workspace(need, values.device)
+    init_c = _CTYPE[code](init)
+    fn = lib().mgpu_hip_segreduce_phases
+    args = (_ptr(values), count, _ptr(segments), nseg, _ptr(out), code, OPS[op],
+            ctypes.byref(init_c), _ptr(ws), ws.numel(), _stream(), phases)
+    keep = (values, segments, out, ws, init_c)      # what the pointers point at
+
+    def call():
+        _check(fn(*args))
+        return keep[2]
+    return call, out
+
+
+def prepare_load_balance_search(count, segments, out=None, phases=3):
+    """load_balance_search() prepared the same way."""
+    _dev_i32(segments, "segments")
+    nseg = segments.numel()
+    if out is None:
+        out = torch.empty(count, dtype=torch.int32, device=segments.device)
+    ws = _workspace(lib().mgpu_hip_lbs_workspace_bytes(count, nseg), segments.device)
+    fn = lib().mgpu_hip_load_balance_search_phases
+    args = (count, _ptr(segments), nseg, _ptr(out), _ptr(ws), ws.numel(), _stream(), phases)
+    keep = (segments, out, ws)
+
+    def call():
+        _check(fn(*args))
+        return keep[1]
+    return call, out
+
+
 def transform_segreduce_mod13(count, segments, init=-1, out=None):
     """transform_segreduce with f(index) = index % 13, int32 plus."""
     _dev_i32(segments, "segments")
