@@ -222,3 +222,25 @@ def test_lbs_segreduce_seg_plus_rank(oracle, dev):
         got = m.lbs_segreduce_seg_plus_rank(count, _dev(segs), init=-1)
         want = oracle.lbs_segreduce_seg_plus_rank(count, segs, init=-1)
         assert np.array_equal(got.cpu().numpy(), want), (count, nseg)
+
+
+def test_prepared_calls_match_direct_calls(oracle, dev):
+    """prepare_segreduce / prepare_load_balance_search marshal the arguments
+    once; what they enqueue must be the ordinary call."""
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    w = workloads.config1(count=300_000, num_segments=4_000)
+    values, segs = torch.from_numpy(w["values"]).to(dev), torch.from_numpy(w["segments"]).to(dev)
+    call, out = m.prepare_segreduce(values, segs, "plus", 0)
+    for _ in range(3):
+        out.fill_(-7)
+        assert call() is out
+        torch.cuda.synchronize()
+        assert np.array_equal(out.cpu().numpy(),
+                              oracle.segreduce(w["values"], w["segments"], "plus", 0))
+    call, out = m.prepare_load_balance_search(300_000, segs)
+    call()
+    torch.cuda.synchronize()
+    assert np.array_equal(out.cpu().numpy(),
+                          oracle.load_balance_search(300_000, w["segments"]))
