@@ -124,7 +124,7 @@ void interval_expand(input_it input, int count, segments_it segments,
   typedef typename std::iterator_traits<input_it>::value_type type_t;
   detail::interval_expand_f<type_t, output_it> fill { output };
   transform_lbs<launch_arg_t>(fill, count, segments, num_segments,
-    make_tuple(input), context);
+    mgpu::make_tuple(input), context);
 }
 
 // Segment s reads its items from input starting at gather[s]:
@@ -136,7 +136,7 @@ void interval_gather(input_it input, int count, segments_it segments,
   typename detail::interval_copy_select_t<false, true, input_it,
     output_it>::type copy { input, output };
   transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
-    make_tuple(gather), context);
+    mgpu::make_tuple(gather), context);
 }
 
 // Segment s writes its items to output starting at scatter[s]:
@@ -149,7 +149,7 @@ void interval_scatter(input_it input, int count, segments_it segments,
   typename detail::interval_copy_select_t<true, false, input_it,
     output_it>::type copy { input, output };
   transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
-    make_tuple(scatter), context);
+    mgpu::make_tuple(scatter), context);
 }
 
 // Both at once: output[scatter[s] + rank] = input[gather[s] + rank].
@@ -162,7 +162,7 @@ void interval_move(input_it input, int count, segments_it segments,
   typename detail::interval_copy_select_t<true, true, input_it,
     output_it>::type copy { input, output };
   transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
-    make_tuple(scatter, gather), context);
+    mgpu::make_tuple(scatter, gather), context);
 }
 
 END_MGPU_NAMESPACE

@@ -60,7 +60,8 @@ mem_t<int2> inner_join(a_it a, int a_count, b_it b, int b_count,
 
   mem_t<int2> output(join_count, context);
   transform_lbs<launch_arg_t>(detail::join_pairs_f { output.data() },
-    join_count, starts.data(), a_count, make_tuple(lower_data), context);
+    join_count, starts.data(), a_count, mgpu::make_tuple(lower_data),
+    context);
   return output;
 }
 

@@ -4,6 +4,7 @@
 // the mgpu:: API, and the context's allocator hooks.  Non-zero exit on error.
 #include <moderngpu/kernel_segreduce.hxx>
 #include <moderngpu/kernel_intervalmove.hxx>
+#include <moderngpu/kernel_scan.hxx>
 #include <cstdio>
 #include <cmath>
 
@@ -232,7 +233,66 @@ int main() {
     context.synchronize();
   }
 
-  // 7. timer and properties.
+  // 7. iterators that are not pointers on every side: segment starts through
+  // a load iterator, values from a counting iterator, results through a
+  // load/store iterator; the search stored through a store iterator; scan
+  // into a store iterator.
+  {
+    int count = 180001, num_segments = 3000;
+    std::vector<int> seg_host = make_segments(count, num_segments, 23);
+    mem_t<int> segments = to_mem(seg_host, context);
+    const int* seg_data = segments.data();
+    auto seg_it = make_load_iterator<int>(
+      [=]MGPU_DEVICE(int i) { return seg_data[i]; });
+
+    mem_t<int64_t> results(num_segments, context);
+    int64_t* res_data = results.data();
+    auto res_it = make_load_store_iterator<int64_t>(
+      [=]MGPU_DEVICE(int i) { return res_data[i] - 5; },
+      [=]MGPU_DEVICE(int64_t x, int i) { res_data[i] = x + 5; });
+    segreduce(counting_iterator_t<int64_t>(0), count, seg_it, num_segments,
+      res_it, plus_t<int64_t>(), (int64_t)-9, context);
+    std::vector<int64_t> got = from_mem(results);
+    for(int s = 0; s < num_segments; ++s) {
+      int64_t b = seg_host[s], e = s + 1 < num_segments ? seg_host[s + 1] : count;
+      int64_t want = e > b ? (e - 1) * e / 2 - (b - 1) * b / 2 : -9;
+      CHECK(got[s] == want + 5);
+    }
+
+    mem_t<int> found(count, context);
+    int* found_data = found.data();
+    load_balance_search(count, seg_it, num_segments, make_store_iterator<int>(
+      [=]MGPU_DEVICE(int seg, int i) { found_data[i] = 2 * seg + 1; }), context);
+    std::vector<int> f = from_mem(found);
+    int seg = -1;
+    for(int i = 0; i < count; ++i) {
+      while(seg + 1 < num_segments && seg_host[seg + 1] <= i) ++seg;
+      CHECK(f[i] == 2 * seg + 1);
+    }
+
+    mem_t<float> expanded(count, context);
+    interval_expand(strided_iterator_t<int>(7, 3), count, seg_it,
+      num_segments, expanded.data(), context);
+    std::vector<float> ex = from_mem(expanded);
+    seg = -1;
+    for(int i = 0; i < count; ++i) {
+      while(seg + 1 < num_segments && seg_host[seg + 1] <= i) ++seg;
+      CHECK(ex[i] == (float)(7 + 3 * seg));
+    }
+
+    mem_t<int> scanned(count, context);
+    int* scanned_data = scanned.data();
+    mem_t<int> total(1, context);
+    scan(counting_iterator_t<int>(0), count, make_store_iterator<int>(
+      [=]MGPU_DEVICE(int x, int i) { scanned_data[i] = x ^ 1; }),
+      plus_t<int>(), total.data(), context);
+    std::vector<int> sc = from_mem(scanned);
+    for(int i = 0; i < count; ++i)
+      CHECK(sc[i] == ((int)((int64_t)i * (i - 1) / 2) ^ 1));
+    CHECK(from_mem(total)[0] == (int)((int64_t)count * (count - 1) / 2));
+  }
+
+  // 8. timer and properties.
   context.timer_begin();
   double seconds = context.timer_end();
   CHECK(seconds >= 0);
