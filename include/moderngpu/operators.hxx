@@ -73,9 +73,24 @@ MGPU_DEF_BINARY(minimum_t, type_t, mgpu::min(a, b))
     moved.member -= n; return moved;                                          \
   }
 
+// The member types std::iterator_traits looks for, as those of a pointer to
+// const.  They are spelled out instead of inherited from
+// std::iterator_traits<const value_type*>: a base class from namespace std
+// would make std an associated namespace of every iterator here, and an
+// unqualified make_tuple(...) or get<0>(...) on them ambiguous with the
+// standard library's.
+template<typename value_t>
+struct iterator_types_t {
+  typedef value_t value_type;
+  typedef std::ptrdiff_t difference_type;
+  typedef const value_t* pointer;
+  typedef const value_t& reference;
+  typedef std::random_access_iterator_tag iterator_category;
+};
+
 // CRTP base: a position and the offset operators.
 template<typename outer_t, typename int_t, typename value_type>
-struct iterator_t : std::iterator_traits<const value_type*> {
+struct iterator_t : iterator_types_t<value_type> {
   int_t index;
   iterator_t() = default;
   MGPU_HOST_DEVICE iterator_t(int_t i) : index(i) { }
@@ -151,7 +166,7 @@ struct constant_iterator_t :
 // kernels through make_load_iterator (src/moderngpu/kernel_segreduce.hxx:278).
 
 template<typename load_t, typename store_t, typename value_type, typename int_t>
-struct lambda_iterator_t : std::iterator_traits<const value_type*> {
+struct lambda_iterator_t : iterator_types_t<value_type> {
   enum {
     can_load = !std::is_same<load_t, empty_t>::value,
     can_store = !std::is_same<store_t, empty_t>::value

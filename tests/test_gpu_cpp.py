@@ -49,3 +49,7 @@ def test_workcreate_engine_and_bfs(dev):
 
 def test_reference_style_sorted_search_and_join(dev):
     assert "all passed" in _run("test_join")
+
+
+def test_api_surface_with_iterators_and_wide_types(dev):
+    assert "all passed" in _run("test_api_surface")
