@@ -1,0 +1,195 @@
+// The small pieces user kernels are written with: launch front ends
+// (transform, cta_transform, cta_launch incl. the device-side tile count),
+// tile movement between memory, LDS and registers in both orders, mem_t and
+// its factories, tuples of iterators, compile-time helpers.  Each is checked
+// against a host computation.  Exit status 1 on the first mismatch.
+#include <moderngpu/transform.hxx>
+#include <moderngpu/memory.hxx>
+#include <moderngpu/loadstore.hxx>
+#include <moderngpu/cpp11.hxx>
+#include <cstdio>
+
+using namespace mgpu;
+
+#define CHECK(cond) do { if(!(cond)) { \
+  printf("%s:%d: CHECK(%s) failed\n", __FILE__, __LINE__, #cond); return 1; \
+} } while(0)
+
+static_assert(div_up(10, 3) == 4 && div_up((int64_t)1 << 40, (int64_t)3) > 0, "");
+static_assert(div_up(2147483647, 4096) == 524288, "no overflow at the top");
+static_assert(s_log2(1) == 0 && s_log2(4096) == 12 && s_log2(4097) == 12, "");
+static_assert(is_pow2(64) && !is_pow2(96), "");
+static_assert(mgpu::max(3, 3) == 3 && mgpu::min(2, 5) == 2, "");
+static_assert(tuple_union_size<tuple<char, double, int> >::value == 8, "");
+
+static int check_launches(context_t& context) {
+  int count = 100003;
+  mem_t<int> out = fill<int>(-1, count, context);
+  int* p = out.data();
+  // transform with pass-through arguments
+  transform([]MGPU_DEVICE(int index, int* dest, int scale) {
+    dest[index] = scale * index;
+  }, count, context, p, 3);
+  std::vector<int> host = from_mem(out);
+  for(int i = 0; i < count; ++i) CHECK(host[i] == 3 * i);
+
+  // cta_transform: one CTA per nv items, every thread sees (tid, cta)
+  enum { nt = 128, vt = 5 };
+  cta_transform<nt, vt>([=]MGPU_DEVICE(int tid, int cta) {
+    strided_iterate<nt, vt>([=](int, int j) { p[nt * vt * cta + j] = cta; },
+      tid, count - nt * vt * cta);
+  }, count, context);
+  host = from_mem(out);
+  for(int i = 0; i < count; ++i) CHECK(host[i] == i / (nt * vt));
+
+  // cta_launch with the tile count in device memory
+  int tiles = 777;
+  mem_t<int> num_tiles = to_mem(std::vector<int> { tiles }, context);
+  mem_t<int> hits = fill<int>(0, 1000, context);
+  int* h = hits.data();
+  cta_launch<launch_params_t<64, 1> >([=]MGPU_DEVICE(int tid, int tile) {
+    if(!tid) atomicAdd(h + tile, 1);
+  }, num_tiles.data(), context);
+  host = from_mem(hits);
+  for(int i = 0; i < 1000; ++i) CHECK(host[i] == (i < tiles ? 1 : 0));
+
+  // nothing is launched for zero work
+  cta_launch<nt>([=]MGPU_DEVICE(int, int) { p[0] = 12345; }, 0, context);
+  transform([=]MGPU_DEVICE(int) { p[0] = 12345; }, 0, context);
+  CHECK(from_mem(out)[0] == 0);
+  return 0;
+}
+
+static int check_tile_movement(context_t& context) {
+  enum { nt = 128, vt = 7, nv = nt * vt };
+  int count = 5 * nv + 333;                 // last tile partial
+  int num_ctas = div_up(count, (int)nv);
+  std::vector<int> in_host(count);
+  for(int i = 0; i < count; ++i) in_host[i] = 10 * i + 1;
+  mem_t<int> in = to_mem(in_host, context);
+  mem_t<int> a(count, context), b(count, context), c(count, context),
+    d(count, context);
+  const int* src = in.data();
+  int *pa = a.data(), *pb = b.data(), *pc = c.data(), *pd = d.data();
+
+  cta_launch<nt>([=]MGPU_DEVICE(int tid, int cta) {
+    __shared__ int shared[nv];
+    int base = nv * cta;
+    int n = min((int)nv, count - base);
+
+    // strided load -> thread order -> add the position in thread order ->
+    // back to strided -> store
+    array_t<int, vt> x = mem_to_reg_strided<nt, vt>(src + base, tid, n);
+    array_t<int, vt> y = reg_strided_to_thread<nt, vt>(x, tid, shared);
+    iterate<vt>([&](int i) { y[i] += vt * tid + i; });
+    x = reg_thread_to_strided<nt, vt>(y, tid, shared);
+    reg_to_mem_strided<nt, vt>(x, tid, n, pa + base);
+
+    // thread-order load and store through LDS
+    array_t<int, vt> z = mem_to_reg_thread<nt, vt>(src + base, tid, n, shared);
+    iterate<vt>([&](int i) { z[i] = 2 * z[i]; });
+    reg_to_mem_thread<nt, vt>(z, tid, n, pb + base, shared);
+
+    // memory -> LDS -> gather reversed within the tile -> memory
+    mem_to_shared<nt, vt>(src + base, tid, n, shared);
+    array_t<int, vt> indices;
+    iterate<vt>([&](int i) {
+      int j = nt * i + tid;
+      indices[i] = j < n ? n - 1 - j : 0;
+    });
+    array_t<int, vt> g = shared_gather<nt, vt>(shared, indices);
+    reg_to_mem_strided<nt, vt>(g, tid, n, pc + base);
+
+    // straight copy
+    mem_to_mem<nt, vt>(src + base, tid, n, pd + base);
+  }, num_ctas, context);
+
+  std::vector<int> ha = from_mem(a), hb = from_mem(b), hc = from_mem(c),
+    hd = from_mem(d);
+  for(int i = 0; i < count; ++i) {
+    int base = i / nv * nv, n = std::min((int)nv, count - base);
+    CHECK(ha[i] == in_host[i] + (i - base));
+    CHECK(hb[i] == 2 * in_host[i]);
+    CHECK(hc[i] == in_host[base + n - 1 - (i - base)]);
+    CHECK(hd[i] == in_host[i]);
+  }
+  return 0;
+}
+
+static int check_memory(context_t& context) {
+  int count = 4099;
+  mem_t<double> halves = fill_function<double>(
+    []MGPU_DEVICE(int i) { return 0.5 * i; }, count, context);
+  mem_t<double> copy = halves.clone();
+  CHECK(copy.data() != halves.data() && copy.size() == halves.size());
+  std::vector<double> h = from_mem(copy);
+  for(int i = 0; i < count; ++i) CHECK(h[i] == 0.5 * i);
+
+  mem_t<int64_t> counted = copy_to_mem(counting_iterator_t<int64_t>(7), count,
+    context);
+  std::vector<int64_t> c = from_mem(counted);
+  for(int i = 0; i < count; ++i) CHECK(c[i] == 7 + i);
+
+  mem_t<int64_t> second(count, context);
+  CHECK(hipSuccess == dtod(second.data(), counted.data(), count));
+  std::vector<int64_t> back(3);
+  CHECK(hipSuccess == dtoh(back, second.data() + 10, 3));
+  CHECK(back.size() == 3 && back[0] == 17 && back[2] == 19);
+  std::vector<int64_t> elsewhere(3);
+  CHECK(hipSuccess == htoh(elsewhere.data(), back.data(), 3));
+  CHECK(elsewhere == back);
+  CHECK(hipSuccess == htod(second.data(), elsewhere));
+  CHECK(from_mem(second)[1] == 18);
+
+  // pinned host memory, move semantics
+  mem_t<int> pinned(16, context, memory_space_host);
+  CHECK(memory_space_host == pinned.space());
+  pinned.data()[3] = 42;
+  mem_t<int> moved = std::move(pinned);
+  CHECK(moved.data()[3] == 42 && pinned.data() == nullptr);
+
+  mem_t<int> sorted = fill_random(0, 1000, 5000, true, context);
+  std::vector<int> s = from_mem(sorted);
+  CHECK(std::is_sorted(s.begin(), s.end()) && s.front() >= 0 && s.back() <= 1000);
+  return 0;
+}
+
+static int check_tuples(context_t& context) {
+  // host side
+  tuple<int, double, char> t = make_tuple(3, 2.5, 'x');
+  CHECK(get<0>(t) == 3 && get<1>(t) == 2.5 && get<2>(t) == 'x');
+  CHECK(make_tuple(1, 2) < make_tuple(1, 3) && make_tuple(2, 0) > make_tuple(1, 9));
+  CHECK(make_tuple(4, 4) == make_tuple(4, 4) && make_tuple(4, 4) != make_tuple(4, 5));
+  CHECK(make_tuple(1, 2) <= make_tuple(1, 2) && make_tuple(1, 2) >= make_tuple(1, 2));
+
+  // device side: tuples of iterators read and written as one
+  int count = 3001;
+  mem_t<int> a(count, context);
+  mem_t<float> b(count, context);
+  mem_t<int> sum(count, context);
+  auto outputs = make_tuple(a.data(), b.data());
+  int* s = sum.data();
+  transform([=]MGPU_DEVICE(int i) {
+    store(outputs, make_tuple(i, 0.25f * i), i);
+  }, count, context);
+  transform([=]MGPU_DEVICE(int i) {
+    tuple<int, float> v = load(outputs, i);
+    get<0>(dereference(outputs, i)) += 1;         // a reference into a[]
+    s[i] = get<0>(v) + (int)(4 * get<1>(v));
+  }, count, context);
+  std::vector<int> ha = from_mem(a), hs = from_mem(sum);
+  std::vector<float> hb = from_mem(b);
+  for(int i = 0; i < count; ++i)
+    CHECK(ha[i] == i + 1 && hb[i] == 0.25f * i && hs[i] == 2 * i);
+  return 0;
+}
+
+int main() {
+  standard_context_t context(false);
+  CHECK(0 == check_launches(context));
+  CHECK(0 == check_tile_movement(context));
+  CHECK(0 == check_memory(context));
+  CHECK(0 == check_tuples(context));
+  printf("runtime: all passed\n");
+  return 0;
+}

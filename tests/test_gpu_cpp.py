@@ -53,3 +53,7 @@ def test_reference_style_sorted_search_and_join(dev):
 
 def test_api_surface_with_iterators_and_wide_types(dev):
     assert "all passed" in _run("test_api_surface")
+
+
+def test_runtime_helpers(dev):
+    assert "all passed" in _run("test_runtime")
