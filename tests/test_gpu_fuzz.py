@@ -1,0 +1,101 @@
+"""Many small random shapes through the C ABI against the CPU checker: sizes
+around one to a few tiles, segment starts with heavy duplication (runs of
+empty segments), starts equal to count, single segments, no items.  Integer
+types only, so everything must match bit for bit.  The seeds are fixed: a
+failure names its case."""
+import numpy as np
+import pytest
+import torch
+
+pytestmark = pytest.mark.gpu
+
+SIZES = [0, 1, 2, 63, 64, 65, 255, 256, 257, 2047, 2048, 2049, 4095, 4096, 4097,
+         6079, 6080, 6081, 6143, 6144, 6145, 8191, 8192, 12287, 12288, 20000, 50001]
+
+
+def _case(rng):
+    count = int(rng.choice(SIZES)) + int(rng.integers(0, 3))
+    kind = int(rng.integers(0, 6))
+    if kind == 0:
+        nseg = 1
+    elif kind == 1:
+        nseg = int(rng.integers(1, 8))
+    elif kind == 2:
+        nseg = max(1, count // int(rng.integers(1, 40)))
+    elif kind == 3:
+        nseg = count + int(rng.integers(1, 300))          # more segments than items
+    elif kind == 4:
+        nseg = int(rng.integers(1, 5000))
+    else:
+        nseg = int(rng.choice(SIZES)) + 1
+    starts = np.zeros(nseg, dtype=np.int32)
+    if nseg > 1:
+        draws = rng.integers(0, count + 1, size=nseg - 1)
+        mode = int(rng.integers(0, 4))
+        if mode == 1:                                     # few distinct starts
+            draws = rng.choice(rng.integers(0, count + 1, size=4), size=nseg - 1)
+        elif mode == 2:                                   # everything at the end
+            draws[:] = count
+        elif mode == 3:                                   # on multiples of 64
+            draws = (draws // 64) * 64
+        starts[1:] = np.sort(draws)
+    return count, starts
+
+
+@pytest.mark.parametrize("seed", range(40))
+def test_segreduce_lbs_scan_fuzz(oracle, dev, seed):
+    import moderngpu_amd as m
+    rng = np.random.default_rng(1000 + seed)
+    for _ in range(6):
+        count, starts = _case(rng)
+        tag = (seed, count, starts.size)
+        segs = torch.from_numpy(starts).to(dev)
+        dtype = [np.int32, np.int64][int(rng.integers(0, 2))]
+        op = ["plus", "maximum", "minimum"][int(rng.integers(0, 3))]
+        values = rng.integers(-1000, 1000, size=count).astype(dtype)
+        got = m.segreduce(torch.from_numpy(values).to(dev), segs, op, -77)
+        assert np.array_equal(got.cpu().numpy(),
+                              oracle.segreduce(values, starts, op, -77)), ("segreduce",) + tag
+        got = m.load_balance_search(count, segs)
+        want = oracle.load_balance_search(count, starts)
+        assert np.array_equal(got.cpu().numpy(), want), ("lbs",) + tag
+        seg, rank = m.transform_lbs(count, segs)
+        assert np.array_equal(seg.cpu().numpy(), want), ("transform_lbs seg",) + tag
+        assert np.array_equal(rank.cpu().numpy(),
+                              np.arange(count, dtype=np.int64) - starts[want].astype(np.int64)
+                              if count else np.zeros(0)), ("transform_lbs rank",) + tag
+        per_seg = rng.integers(0, 1 << 20, size=starts.size).astype(np.int32)
+        got = m.interval_expand(torch.from_numpy(per_seg).to(dev), count, segs)
+        assert np.array_equal(got.cpu().numpy(),
+                              oracle.interval_expand(per_seg, count, starts)), ("expand",) + tag
+        got, _ = m.scan(torch.from_numpy(values).to(dev), op, inclusive=bool(seed & 1))
+        assert np.array_equal(got.cpu().numpy(),
+                              oracle.scan(values, op, 0, inclusive=bool(seed & 1))[0]), \
+            ("scan",) + tag
+        created = rng.integers(-1, 4, size=count).astype(np.int32)
+        got = m.workcreate(torch.from_numpy(created).to(dev), segs)
+        want = oracle.workcreate(created, starts)
+        assert got[0] == want[0], ("workcreate count",) + tag
+        for g, x in zip(got[1:], want[1:]):
+            assert np.array_equal(g.cpu().numpy(), x), ("workcreate",) + tag
+
+
+@pytest.mark.parametrize("seed", range(20))
+def test_search_and_join_fuzz(oracle, dev, seed):
+    import moderngpu_amd as m
+    rng = np.random.default_rng(2000 + seed)
+    for _ in range(6):
+        n = int(rng.choice(SIZES[:22])) + int(rng.integers(0, 3))
+        h = int(rng.choice(SIZES[:22])) + int(rng.integers(0, 3))
+        hi = int(rng.choice([0, 1, 5, 100, 10000, 1 << 30]))
+        a = np.sort(rng.integers(0, hi + 1, size=n)).astype(np.int32)
+        b = np.sort(rng.integers(0, hi + 1, size=h)).astype(np.int32)
+        da, db = torch.from_numpy(a).to(dev), torch.from_numpy(b).to(dev)
+        for bounds in ("lower", "upper"):
+            got = m.sorted_search(da, db, bounds)
+            assert np.array_equal(got.cpu().numpy(),
+                                  oracle.sorted_search(a, b, upper=(bounds == "upper"))), \
+                (seed, n, h, hi, bounds)
+        if n * h < 4_000_000 or hi > 100:
+            got = m.inner_join(da, db)
+            assert np.array_equal(got.cpu().numpy(), oracle.inner_join(a, b)), (seed, n, h, hi)
