@@ -199,8 +199,77 @@ static int check_scans(context_t& context) {
   return 0;
 }
 
+// Every algorithm under a caller's launch box, from one wavefront with one
+// item per thread to 1,024 threads.
+template<typename box_t>
+static int check_box(context_t& context) {
+  int count = 70003, num_segments = 900;
+  std::vector<int> seg_host = make_segments(count, num_segments, 61);
+  mem_t<int> segments = to_mem(seg_host, context);
+  std::vector<int> v(count);
+  std::mt19937 mt(62);
+  for(int& x : v) x = (int)(mt() % 2001) - 1000;
+  mem_t<int> values = to_mem(v, context);
+
+  mem_t<int> scanned(count, context), total(1, context);
+  scan<scan_type_exc, box_t>(values.data(), count, scanned.data(), plus_t<int>(),
+    total.data(), context);
+  std::vector<int> sc = from_mem(scanned);
+  int run = 0;
+  for(int i = 0; i < count; ++i) { CHECK(sc[i] == run); run += v[i]; }
+  CHECK(from_mem(total)[0] == run);
+
+  mem_t<int> folded(1, context);
+  reduce<box_t>(values.data(), count, folded.data(), maximum_t<int>(), context);
+  CHECK(from_mem(folded)[0] == *std::max_element(v.begin(), v.end()));
+
+  mem_t<int> sums(num_segments, context);
+  lbs_segreduce<box_t>([]MGPU_DEVICE(int index, int seg, int rank,
+    tuple<int> start, const int* values) {
+      return values[index] + (get<0>(start) + rank - index);
+    }, count, segments.data(), num_segments, make_tuple(segments.data()),
+    sums.data(), plus_t<int>(), -1, context, values.data());
+  std::vector<int> got = from_mem(sums);
+  for(int s = 0; s < num_segments; ++s) {
+    int b = seg_host[s], e = s + 1 < num_segments ? seg_host[s + 1] : count;
+    int want = -1;
+    for(int i = b; i < e; ++i) want = (i == b) ? v[i] : want + v[i];
+    CHECK(got[s] == want);
+  }
+
+  // gather each segment from where a reversed layout of the segments put it
+  std::vector<int> base(num_segments);
+  int at = 0;
+  for(int s = num_segments - 1; s >= 0; --s) {
+    base[s] = at;
+    at += (s + 1 < num_segments ? seg_host[s + 1] : count) - seg_host[s];
+  }
+  mem_t<int> bases = to_mem(base, context);
+  mem_t<int> gathered(count, context), moved(count, context);
+  interval_gather<box_t>(values.data(), count, segments.data(), num_segments,
+    bases.data(), gathered.data(), context);
+  interval_move<box_t>(gathered.data(), count, segments.data(), num_segments,
+    bases.data(), segments.data(), moved.data(), context);
+  std::vector<int> g = from_mem(gathered), mv = from_mem(moved);
+  int seg = -1;
+  for(int i = 0; i < count; ++i) {
+    while(seg + 1 < num_segments && seg_host[seg + 1] <= i) ++seg;
+    int rank = i - seg_host[seg];
+    CHECK(g[i] == v[base[seg] + rank]);
+    CHECK(mv[base[seg] + rank] == g[i]);
+  }
+  return 0;
+}
+
 int main() {
   standard_context_t context(false);
+  CHECK(0 == (check_box<launch_params_t<64, 1> >(context)));
+  CHECK(0 == (check_box<launch_params_t<64, 3> >(context)));
+  CHECK(0 == (check_box<launch_params_t<128, 7> >(context)));
+  CHECK(0 == (check_box<launch_params_t<256, 4> >(context)));
+  CHECK(0 == (check_box<launch_params_t<512, 2> >(context)));
+  CHECK(0 == (check_box<launch_params_t<1024, 1> >(context)));
+  CHECK(0 == (check_box<launch_params_t<1024, 8> >(context)));
   CHECK(0 == check_wide_values(context));
   CHECK(0 == check_lbs_with_mixed_cache(context));
   CHECK(0 == check_wide_keys(context));
