@@ -16,6 +16,7 @@ import select
 import subprocess
 import time
 
+import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
@@ -108,3 +109,80 @@ def test_reference_test_join_and_intervalexpand(dev):
     for name in ("test_join", "test_intervalexpand"):
         code, out, err = _run(name)
         assert code == 0, name + err[-2000:]
+
+
+# ---- the breadth-first-search demos (demo/bfs.cu:1-92, bfs2.cu:1-113,
+# bfs3.cu:1-134 with demo/graph.cxx:7-56) ------------------------------------
+# They read a Matrix Market file at a fixed relative path (a graph that the
+# reference does not ship), start at vertex 23, and write the level of every
+# vertex to bfs.txt (bfs, bfs2) or print the size of every front (bfs3).  The
+# tests give them a synthetic graph at that path in a scratch directory and
+# compare with a breadth-first search in numpy.
+
+def _synthetic_graph(tmp_path, num_vertices, num_edges, seed):
+    rng = np.random.default_rng(seed)
+    # A few hubs, many leaves, some vertices that nothing reaches.
+    reach = int(num_vertices * 0.9)
+    a = rng.integers(0, reach, num_edges)
+    b = (rng.zipf(1.6, num_edges) + rng.integers(0, reach, num_edges)) % reach
+    a[0], b[0] = 23, 24                         # the source has a neighbour
+    folder = tmp_path / "demo" / "coPapersCiteseer"
+    folder.mkdir(parents=True)
+    with open(folder / "coPapersCiteseer.mtx", "w") as f:
+        f.write("%%MatrixMarket matrix coordinate pattern symmetric\n")
+        f.write("% synthetic\n")
+        f.write("%d %d %d\n" % (num_vertices, num_vertices, num_edges))
+        f.write("".join("%d %d\n" % (x + 1, y + 1) for x, y in zip(a, b)))
+    # The loader stores every edge in both directions (graph.cxx:22-38).
+    src = np.concatenate([a, b])
+    dst = np.concatenate([b, a])
+    order = np.lexsort((dst, src))
+    src, dst = src[order], dst[order]
+    starts = np.searchsorted(src, np.arange(num_vertices + 1))
+    return starts, dst
+
+
+def _bfs_levels(starts, dst, source):
+    level = np.full(len(starts) - 1, -1, np.int64)
+    level[source] = 0
+    front = np.array([source])
+    fronts = []
+    while len(front):
+        begin, end = starts[front], starts[front + 1]
+        neighbours = np.concatenate([dst[b:e] for b, e in zip(begin, end)]) \
+            if len(front) else np.zeros(0, np.int64)
+        fresh = np.unique(neighbours[level[neighbours] == -1])
+        level[fresh] = level[front[0]] + 1
+        fronts.append((len(fresh), int((starts[fresh + 1] - starts[fresh]).sum())))
+        front = fresh
+    return level, fronts
+
+
+def _run_demo(name, tmp_path):
+    path = os.path.join(BIN, name)
+    if not os.path.exists(path):
+        pytest.skip("reference_callers/%s was not built (no reference tree at build time)" % name)
+    proc = subprocess.run([path], capture_output=True, text=True, timeout=110,
+                          cwd=str(tmp_path))
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    return proc.stdout
+
+
+@pytest.mark.parametrize("name", ["bfs", "bfs2"])
+def test_reference_demo_bfs_levels(dev, tmp_path, name):
+    starts, dst = _synthetic_graph(tmp_path, 60_000, 400_000, 5)
+    want, _ = _bfs_levels(starts, dst, 23)
+    _run_demo(name, tmp_path)
+    got = np.array([int(l.split(":")[1]) for l in open(tmp_path / "bfs.txt")])
+    assert got.shape == want.shape
+    assert (want == -1).any() and want.max() >= 3
+    assert np.array_equal(got, want)
+
+
+def test_reference_demo_bfs3_fronts(dev, tmp_path):
+    starts, dst = _synthetic_graph(tmp_path, 60_000, 400_000, 6)
+    _, fronts = _bfs_levels(starts, dst, 23)
+    out = _run_demo("bfs3", tmp_path)
+    got = [(int(v), int(e)) for v, e in re.findall(
+        r"Front for level \d+ has (\d+) vertices and (\d+) edges", out)]
+    assert got == fronts
