@@ -80,6 +80,17 @@ MGPU_HOST_DEVICE auto dereference(tuple<its_t...> its, int_t index) ->
     make_index_sequence<sizeof...(its_t)>());
 }
 
+// var_max<a, b, ...>::value: the largest of the arguments, 0 for none.
+template<size_t... values>
+struct var_max {
+  constexpr static size_t value = 0;
+};
+template<size_t first, size_t... rest>
+struct var_max<first, rest...> {
+  constexpr static size_t value = first < var_max<rest...>::value ?
+    var_max<rest...>::value : first;
+};
+
 // Size of the largest element type: what a union of them needs.
 template<typename tpl_t>
 struct tuple_union_size;

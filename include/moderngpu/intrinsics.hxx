@@ -58,6 +58,23 @@ MGPU_HOST_DEVICE unsigned prmt(unsigned a, unsigned b, unsigned index) {
   return result;
 }
 
+// Bits of x in reverse order.
+MGPU_HOST_DEVICE unsigned brev(unsigned x) { return __builtin_bitreverse32(x); }
+
+// floor(log2(x)), or ceil(log2(x)) with round_up; x > 0.
+MGPU_HOST_DEVICE int find_log2(int x, bool round_up = false) {
+  int floor_log = 31 - clz(x);
+  return floor_log + (round_up && (x & (x - 1)) ? 1 : 0);
+}
+
+// Upper 32 bits of the 64-bit product.
+MGPU_HOST_DEVICE int mulhi(int a, int b) {
+  return (int)(((long long)a * b) >> 32);
+}
+MGPU_HOST_DEVICE unsigned umulhi(unsigned a, unsigned b) {
+  return (unsigned)(((unsigned long long)a * b) >> 32);
+}
+
 ////////////////////////////////////////////////////////////////////////////////
 // Wavefront queries.
 

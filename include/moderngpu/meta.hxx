@@ -86,6 +86,11 @@ MGPU_HOST_DEVICE constexpr real_t min(real_t a, real_t b) {
   return (b < a) ? b : a;
 }
 
+// Takes any arguments and does nothing: swallow(f(args)...) evaluates a pack
+// expansion for its side effects.
+template<typename... args_t>
+MGPU_HOST_DEVICE void swallow(args_t...) { }
+
 ////////////////////////////////////////////////////////////////////////////////
 // Launch-box plumbing.
 

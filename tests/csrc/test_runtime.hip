@@ -184,8 +184,52 @@ static int check_tuples(context_t& context) {
   return 0;
 }
 
+// The bit helpers on host and device against plain loops.
+static int check_bit_helpers(context_t& context) {
+  static_assert(var_max<3, 9, 4>::value == 9 && var_max<>::value == 0, "");
+  swallow(1, 2.0, "three");
+  const int count = 4096;
+  mem_t<unsigned> out(6 * count, context);
+  unsigned* p = out.data();
+  transform([=]MGPU_DEVICE(int i) {
+    unsigned x = 2654435761u * (unsigned)(i + 1);
+    p[6 * i + 0] = brev(x);
+    p[6 * i + 1] = (unsigned)find_log2((int)(x >> 1) | 1);
+    p[6 * i + 2] = (unsigned)find_log2((int)(x >> 1) | 1, true);
+    p[6 * i + 3] = (unsigned)mulhi((int)x, (int)(x * 7u + 3u));
+    p[6 * i + 4] = umulhi(x, x * 7u + 3u);
+    p[6 * i + 5] = bfi(x, ~x, 5, 9) ^ bfe(x, 7, 11) ^ prmt(x, ~x, 0x5140) ^
+      (unsigned)popc(x) ^ (unsigned)clz(x) ^ (unsigned)ffs(x);
+  }, count, context);
+  std::vector<unsigned> got = from_mem(out);
+  for(int i = 0; i < count; ++i) {
+    unsigned x = 2654435761u * (unsigned)(i + 1);
+    unsigned rev = 0;
+    for(int b = 0; b < 32; ++b) rev |= ((x >> b) & 1) << (31 - b);
+    int v = (int)(x >> 1) | 1, lg = 0;
+    while((1ll << (lg + 1)) <= v) ++lg;
+    int lg_up = lg + (((1ll << lg) != v) ? 1 : 0);
+    unsigned y = x * 7u + 3u;
+    CHECK(got[6 * i + 0] == rev && brev(x) == rev);
+    CHECK(got[6 * i + 1] == (unsigned)lg && find_log2(v) == lg);
+    CHECK(got[6 * i + 2] == (unsigned)lg_up && find_log2(v, true) == lg_up);
+    CHECK(got[6 * i + 3] == (unsigned)(int)(((long long)(int)x * (int)y) >> 32));
+    CHECK(got[6 * i + 4] == (unsigned)(((unsigned long long)x * y) >> 32));
+    CHECK(got[6 * i + 5] == (bfi(x, ~x, 5, 9) ^ bfe(x, 7, 11) ^
+      prmt(x, ~x, 0x5140) ^ (unsigned)popc(x) ^ (unsigned)clz(x) ^
+      (unsigned)ffs(x)));
+  }
+  // Hand values.
+  CHECK(brev(1u) == 0x80000000u && find_log2(1) == 0 && find_log2(5, true) == 3);
+  CHECK(mulhi(-1, 1) == -1 && umulhi(0xffffffffu, 0xffffffffu) == 0xfffffffeu);
+  CHECK(bfe(0xabcd1234u, 8, 8) == 0x12u && bfi(0xffu, 0u, 4, 4) == 0xf0u);
+  CHECK(prmt(0x33221100u, 0x77665544u, 0x7531) == 0x77553311u);
+  return 0;
+}
+
 int main() {
   standard_context_t context(false);
+  CHECK(0 == check_bit_helpers(context));
   CHECK(0 == check_launches(context));
   CHECK(0 == check_tile_movement(context));
   CHECK(0 == check_memory(context));
