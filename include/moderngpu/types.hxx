@@ -77,6 +77,25 @@ struct MGPU_ALIGN(16) merge_range_t {
   MGPU_HOST_DEVICE int total() const { return a_count() + b_count(); }
   MGPU_HOST_DEVICE range_t a_range() const { return { a_begin, a_end }; }
   MGPU_HOST_DEVICE range_t b_range() const { return { b_begin, b_end }; }
+  MGPU_HOST_DEVICE bool a_valid() const { return a_begin < a_end; }
+  MGPU_HOST_DEVICE bool b_valid() const { return b_begin < b_end; }
+
+  // The same two ranges laid out back to back from zero (A, then B): their
+  // positions in an LDS array that holds the tile's keys.
+  MGPU_HOST_DEVICE merge_range_t to_local() const {
+    int na = a_count();
+    return { 0, na, na, na + b_count() };
+  }
+  // What is left behind the split mp0 of cross-diagonal diag ...
+  MGPU_HOST_DEVICE merge_range_t partition(int mp0, int diag) const {
+    return { a_begin + mp0, a_end, b_begin + (diag - mp0), b_end };
+  }
+  // ... and what lies between the splits of two diagonals.
+  MGPU_HOST_DEVICE merge_range_t partition(int mp0, int diag0, int mp1,
+    int diag1) const {
+    return { a_begin + mp0, a_begin + mp1, b_begin + (diag0 - mp0),
+      b_begin + (diag1 - mp1) };
+  }
 };
 
 END_MGPU_NAMESPACE

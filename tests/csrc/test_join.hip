@@ -90,8 +90,71 @@ static int check_join(int a_count, int b_count, int max_key,
   return 0;
 }
 
+// serial_search: a CTA holds both key arrays in LDS, every thread merges vt
+// keys from its merge-path split and reports key, position, source and match
+// bits; the host merges the same arrays with std::merge's tie rules and looks
+// the keys up in the other array.
+template<bounds_t bounds>
+static int check_serial_search(int na, int nb, int max_key, context_t& context) {
+  enum { nt = 128, vt = 5, nv = nt * vt };
+  CHECK(na + nb <= nv);
+  mem_t<int> a = fill_random(0, max_key, na, true, context);
+  mem_t<int> b = fill_random(0, max_key, nb, true, context);
+  mem_t<int> keys(nv, context), where(nv, context), flags(3 * nt, context);
+  const int* a_data = a.data(); const int* b_data = b.data();
+  int* keys_data = keys.data(); int* where_data = where.data();
+  int* flags_data = flags.data();
+  cta_launch<nt>([=]MGPU_DEVICE(int tid, int) {
+    __shared__ int shared[nv + 1];
+    for(int i = tid; i < na; i += nt) shared[i] = a_data[i];
+    for(int i = tid; i < nb; i += nt) shared[na + i] = b_data[i];
+    __syncthreads();
+    merge_range_t tile { 0, na, 0, nb };
+    merge_range_t local = tile.to_local();
+    int diag = min(vt * tid, na + nb);
+    int mp = merge_path<bounds>(shared, local, diag, less_t<int>());
+    merge_range_t mine = local.partition(mp, diag);
+    search_result_t<int, vt> r = serial_search<vt, bounds, true>(shared, mine,
+      0, -na, less_t<int>());
+    for(int i = 0; i < vt; ++i) {
+      keys_data[vt * tid + i] = r.keys[i];
+      where_data[vt * tid + i] = r.indices[i];
+    }
+    flags_data[3 * tid + 0] = r.decisions;
+    flags_data[3 * tid + 1] = r.matches_a;
+    flags_data[3 * tid + 2] = r.matches_b;
+  }, 1, context);
+
+  std::vector<int> ha = from_mem(a), hb = from_mem(b), hk = from_mem(keys),
+    hw = from_mem(where), hf = from_mem(flags);
+  int ia = 0, ib = 0;
+  for(int p = 0; p < na + nb; ++p) {
+    bool take_a;
+    if(ia >= na) take_a = false;
+    else if(ib >= nb) take_a = true;
+    else take_a = (bounds_upper == bounds) ? ha[ia] < hb[ib] : !(hb[ib] < ha[ia]);
+    int key = take_a ? ha[ia] : hb[ib];
+    int at = take_a ? ia : ib;
+    bool match = take_a ? std::binary_search(hb.begin(), hb.end(), key) :
+      std::binary_search(ha.begin(), ha.end(), key);
+    int tid = p / vt, i = p % vt;
+    CHECK(hk[p] == key && hw[p] == at);
+    CHECK(((hf[3 * tid + 0] >> i) & 1) == (int)take_a);
+    CHECK(((hf[3 * tid + 1] >> i) & 1) == (int)(take_a && match));
+    CHECK(((hf[3 * tid + 2] >> i) & 1) == (int)(!take_a && match));
+    if(take_a) ++ia; else ++ib;
+  }
+  return 0;
+}
+
 int main() {
   standard_context_t context(false);
+  CHECK(0 == check_serial_search<bounds_lower>(300, 340, 200, context));
+  CHECK(0 == check_serial_search<bounds_upper>(300, 340, 200, context));
+  CHECK(0 == check_serial_search<bounds_lower>(100, 500, 10000, context));
+  CHECK(0 == check_serial_search<bounds_upper>(520, 17, 30, context));
+  CHECK(0 == check_serial_search<bounds_lower>(0, 64, 30, context));
+  CHECK(0 == check_serial_search<bounds_upper>(64, 0, 30, context));
   typedef launch_box_t<arch_20_cta<128, 15>, arch_35_cta<128, 11>,
     arch_52_cta<128, 15> > box_cuda_t;        // the reference's default
   CHECK(0 == check_search<empty_t>(1000, 1000, 10000, context));
