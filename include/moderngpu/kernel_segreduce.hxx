@@ -35,6 +35,7 @@
 #include "search.hxx"
 #include "cta_load_balance.hxx"
 #include "cta_segscan.hxx"
+#include "cta_segreduce.hxx"
 #include "cta_reduce.hxx"
 #include "transform.hxx"
 #include "memory.hxx"

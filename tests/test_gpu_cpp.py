@@ -57,3 +57,7 @@ def test_api_surface_with_iterators_and_wide_types(dev):
 
 def test_runtime_helpers(dev):
     assert "all passed" in _run("test_runtime")
+
+
+def test_caller_built_segreduce_from_cta_blocks(dev):
+    assert "all passed" in _run("test_cta_segreduce")
