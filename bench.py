@@ -374,8 +374,12 @@ def make_c1(copies):
     wk.items = n
     wk.bytes = n * 4 + s * 4 + s * 4
     wk.kernel = "segreduce_tile_f<256x16, int, plus>"
-    wk.step = lambda i: m.segreduce(vals, segs, "plus", 0, out=out)
-    wk.tiles = lambda i: m.segreduce(vals, segs, "plus", 0, out=out, phases=2)
+    # At this size the Python side of an unprepared call (argument checks,
+    # ctypes conversion) costs more than the three kernels.
+    call = m.prepare_segreduce(vals, segs, "plus", 0, out=out)[0]
+    tiles = m.prepare_segreduce(vals, segs, "plus", 0, out=out, phases=2)[0]
+    wk.step = lambda i: call()
+    wk.tiles = lambda i: tiles()
     wk.check = lambda: bool(np.array_equal(
         wk.step(0).cpu().numpy(), oracle.segreduce(w["values"], w["segments"], "plus", 0)))
     wk.cpu = lambda: (lambda: oracle.segreduce(w["values"], w["segments"], "plus", 0))
