@@ -497,7 +497,7 @@ TRAFFIC_BYTES = {
     # + WRITE 4,255.6 KiB x 1.000
     "c2_segreduce_f32": int((134994.4 * 2.000 + 4255.6) * 1024),
     # profiles/transform_lbs_f__c3_load_balance_search.md
-    "c3_load_balance_search": int((33532.2 * 2.000 + 1048576.1) * 1024),
+    "c3_load_balance_search": int((33707.7 * 2.000 + 1048576.1) * 1024),
 }
 
 

@@ -368,10 +368,44 @@ struct cta_load_balance_t {
     return range;
   }
 
+  // The segment starts of a tile read ahead of time into registers (a CTA
+  // that decodes several tiles issues the reads for all of them before it
+  // works on the first).  Tiles with more than prefetch_rows * nt starts are
+  // not read ahead; fill() then reads them itself.
+  enum { prefetch_rows = 2 };
+  struct prefetch_t {
+    int starts[prefetch_rows];
+    int preceding;          // start of the segment open at the tile's begin
+    bool valid;
+  };
+
+  template<typename segments_it>
+  MGPU_DEVICE static prefetch_t prefetch(merge_range_t range,
+    segments_it segments, int tid) {
+    prefetch_t ahead = prefetch_t();
+    int b_count = range.b_count();
+    ahead.valid = b_count <= prefetch_rows * nt;
+    if(ahead.valid) {
+      PRAGMA_UNROLL
+      for(int r = 0; r < prefetch_rows; ++r)
+        if(nt * r + tid < b_count)
+          ahead.starts[r] = segments[range.b_begin + nt * r + tid];
+      if(!tid && range.b_begin) ahead.preceding = segments[range.b_begin - 1];
+    }
+    return ahead;
+  }
+
   // Same for a tile whose range the caller has worked out.
   template<typename segments_it>
   MGPU_DEVICE void fill(merge_range_t range, segments_it segments, int tid,
     storage_t& storage) const {
+    fill(range, segments, tid, storage, prefetch_t());
+  }
+
+  // ... and whose starts the caller may have read ahead with prefetch().
+  template<typename segments_it>
+  MGPU_DEVICE void fill(merge_range_t range, segments_it segments, int tid,
+    storage_t& storage, prefetch_t ahead) const {
 
     int a_count = range.a_count();
     int b_count = range.b_count();
@@ -390,9 +424,16 @@ struct cta_load_balance_t {
     }
 
     // 2. stage the segment starts of the tile.
-    for(int j = tid; j < b_count; j += nt)
-      starts[1 + j] = segments[range.b_begin + j];
-    if(!tid) starts[0] = range.b_begin ? segments[range.b_begin - 1] : 0;
+    if(ahead.valid) {
+      PRAGMA_UNROLL
+      for(int r = 0; r < prefetch_rows; ++r)
+        if(nt * r + tid < b_count) starts[1 + nt * r + tid] = ahead.starts[r];
+      if(!tid) starts[0] = ahead.preceding;
+    } else {
+      for(int j = tid; j < b_count; j += nt)
+        starts[1 + j] = segments[range.b_begin + j];
+      if(!tid) starts[0] = range.b_begin ? segments[range.b_begin - 1] : 0;
+    }
     __syncthreads();
 
     // 3. one marker per segment that owns items here.  Starts ascend, so

@@ -22,6 +22,8 @@ struct interval_expand_f {
 template<typename type_t>
 struct interval_expand_f<type_t, type_t*> {
   typedef void chunk_functor_tag;
+  enum { lbs_tiles_per_cta = 2 };   // two reads, then only stores: see
+                                    // lbs_tiles_per_cta_t
   type_t* output;
   MGPU_DEVICE void operator()(int index, int, int,
     tuple<type_t> desc) const {
