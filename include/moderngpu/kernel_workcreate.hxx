@@ -107,11 +107,14 @@ struct workcreate_tile_t {
   MGPU_DEVICE decoded_t decode(int tid, int tile, storage_t& shared) const {
     merge_range_t range = paired_tile_range(count, num_segments, tile,
       load_balance_t::nv, pairs);
-    // The cached values' read is in flight while the tile is decoded.
+    // The reads of the tile's starts and cached values are issued before
+    // anything waits and land while the tile is decoded.
+    typename load_balance_t::prefetch_t ahead =
+      load_balance_t::prefetch(range, segments, tid);
     value_t fetched;
     bool staged = cached_load_t::fetch(tid, range.b_begin - 1,
       range.b_count() + 1, caching_iterators, fetched);
-    load_balance_t().fill(range, segments, tid, shared.lbs);
+    load_balance_t().fill(range, segments, tid, shared.lbs, ahead);
     cached_load_t::commit(tid, range.b_begin - 1, range.b_count() + 1,
       fetched, shared.cached);
     return decoded_t { range, staged };
