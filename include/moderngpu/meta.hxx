@@ -29,6 +29,10 @@
 #ifndef MGPU_LAMBDA
   #define MGPU_LAMBDA __device__
 #endif
+#ifndef M_PI
+  #define M_PI 3.14159265358979323846
+#endif
+
 #ifndef PRAGMA_UNROLL
   #define PRAGMA_UNROLL _Pragma("unroll")
 #endif
@@ -148,6 +152,20 @@ MGPU_HOST_DEVICE void iterate(func_t f) {
 template<int count, typename func_t>
 MGPU_HOST_DEVICE void iterate(func_t f) {
   iterate<0, count>(f);
+}
+
+// Sum of a small array, and the same value into each of its elements.
+template<int count, typename type_t>
+MGPU_HOST_DEVICE type_t reduce(const type_t (&x)[count]) {
+  type_t sum = x[0];
+  PRAGMA_UNROLL
+  for(int i = 1; i < count; ++i) sum = x[i] + sum;
+  return sum;
+}
+template<int count, typename type_t>
+MGPU_HOST_DEVICE void fill(type_t (&x)[count], type_t value) {
+  PRAGMA_UNROLL
+  for(int i = 0; i < count; ++i) x[i] = value;
 }
 
 ////////////////////////////////////////////////////////////////////////////////

@@ -98,4 +98,17 @@ struct MGPU_ALIGN(16) merge_range_t {
   }
 };
 
+// Register arrays handed between the steps of a merge: keys with values, and
+// keys with the positions they came from.
+template<typename key_t, typename val_t, int size>
+struct kv_array_t {
+  array_t<key_t, size> keys;
+  array_t<val_t, size> vals;
+};
+template<typename type_t, int size>
+struct merge_pair_t {
+  array_t<type_t, size> keys;
+  array_t<int, size> indices;
+};
+
 END_MGPU_NAMESPACE

@@ -188,6 +188,16 @@ static int check_tuples(context_t& context) {
 static int check_bit_helpers(context_t& context) {
   static_assert(var_max<3, 9, 4>::value == 9 && var_max<>::value == 0, "");
   swallow(1, 2.0, "three");
+  {
+    int small[5];
+    mgpu::fill(small, 7);
+    small[2] = -3;
+    CHECK(mgpu::reduce(small) == 25);
+    kv_array_t<int, float, 3> kv; kv.keys[1] = 4; kv.vals[1] = 0.5f;
+    merge_pair_t<short, 2> pair; pair.keys[0] = 9; pair.indices[0] = 1;
+    CHECK(kv.keys[1] == 4 && kv.vals[1] == 0.5f && pair.keys[0] == 9 &&
+      pair.indices[0] == 1 && M_PI > 3.14);
+  }
   const int count = 4096;
   mem_t<unsigned> out(6 * count, context);
   unsigned* p = out.data();
