@@ -147,8 +147,62 @@ static int check_serial_search(int na, int nb, int max_key, context_t& context) 
   return 0;
 }
 
+// A key/value merge assembled from cta_merge_from_mem (which stands on
+// load_two_streams_shared, merge_path and serial_merge) and
+// transfer_two_streams_strided, with merge_path_partitions for the tiles --
+// the way a merge kernel is put together from the CTA-level blocks (moderngpu
+// src/moderngpu/kernel_merge.hxx:30-71).  Values identify where a key came
+// from (a: its index, b: -1 - index), so the order of equal keys is checked
+// too: a stable merge takes equal keys from a first.
+template<int nt, int vt>
+static int check_cta_merge(int na, int nb, int max_key, context_t& context) {
+  enum { nv = nt * vt };
+  mem_t<int> a = fill_random(0, max_key, na, true, context);
+  mem_t<int> b = fill_random(0, max_key, nb, true, context);
+  mem_t<int> a_vals(na, context), b_vals(nb, context);
+  mem_t<int> keys(na + nb, context), vals(na + nb, context);
+  int* av = a_vals.data(); int* bv = b_vals.data();
+  transform([=]MGPU_DEVICE(int i) { av[i] = i; }, na, context);
+  transform([=]MGPU_DEVICE(int i) { bv[i] = -1 - i; }, nb, context);
+  mem_t<int> mp = merge_path_partitions<bounds_lower>(a.data(), na, b.data(),
+    nb, nv, less_t<int>(), context);
+  const int* a_keys = a.data(); const int* b_keys = b.data();
+  const int* mp_data = mp.data();
+  int* c_keys = keys.data(); int* c_vals = vals.data();
+  int num_ctas = div_up(na + nb, (int)nv);
+  cta_launch<nt>([=]MGPU_DEVICE(int tid, int cta) {
+    __shared__ union { int keys[nv + 1]; int indices[nv]; } shared;
+    merge_range_t range = compute_merge_range(na, nb, cta, nv, mp_data[cta],
+      mp_data[cta + 1]);
+    merge_pair_t<int, vt> merged = cta_merge_from_mem<bounds_lower, nt, vt>(
+      a_keys, b_keys, range, tid, less_t<int>(), shared.keys);
+    reg_to_mem_thread<nt>(merged.keys, tid, range.total(), c_keys + nv * cta,
+      shared.keys);
+    array_t<int, vt> where = reg_thread_to_strided<nt>(merged.indices, tid,
+      shared.indices);
+    transfer_two_streams_strided<nt>(av + range.a_begin, range.a_count(),
+      bv + range.b_begin, range.b_count(), where, tid, c_vals + nv * cta);
+  }, num_ctas, context);
+
+  std::vector<int> ha = from_mem(a), hb = from_mem(b), hk = from_mem(keys),
+    hv = from_mem(vals);
+  int ia = 0, ib = 0;
+  for(int p = 0; p < na + nb; ++p) {
+    bool take_a = ia < na && (ib >= nb || !(hb[ib] < ha[ia]));
+    CHECK(hk[p] == (take_a ? ha[ia] : hb[ib]));
+    CHECK(hv[p] == (take_a ? ia : -1 - ib));
+    if(take_a) ++ia; else ++ib;
+  }
+  return 0;
+}
+
 int main() {
   standard_context_t context(false);
+  CHECK(0 == (check_cta_merge<128, 7>(100000, 130000, 5000, context)));
+  CHECK(0 == (check_cta_merge<64, 4>(3000, 50, 40, context)));
+  CHECK(0 == (check_cta_merge<256, 3>(1, 70000, 1 << 30, context)));
+  CHECK(0 == (check_cta_merge<128, 7>(896 * 5, 896 * 3, 100, context)));
+  CHECK(0 == (check_cta_merge<128, 5>(0, 1000, 100, context)));
   CHECK(0 == check_serial_search<bounds_lower>(300, 340, 200, context));
   CHECK(0 == check_serial_search<bounds_upper>(300, 340, 200, context));
   CHECK(0 == check_serial_search<bounds_lower>(100, 500, 10000, context));
