@@ -54,10 +54,13 @@ MGPU_HIP_API int mgpu_hip_version(void);
 /* Text for a return code (hipGetErrorString). */
 MGPU_HIP_API const char* mgpu_hip_error_string(int code);
 /* Merged elements (items + segment starts) between consecutive tile splits:
- * what the library uses as `spacing` for segreduce on `dtype`, and for the
- * load-balancing search. */
+ * what the library uses as `spacing` for segreduce on `dtype`, for the
+ * load-balancing-search kernels that carry per-segment values (interval
+ * expand / gather / scatter / move; the workspace is sized for this one), and
+ * for those that do not (load_balance_search, transform_lbs: larger tiles). */
 MGPU_HIP_API int mgpu_hip_segreduce_tile_size(int dtype);
 MGPU_HIP_API int mgpu_hip_lbs_tile_size(void);
+MGPU_HIP_API int mgpu_hip_lbs_search_tile_size(void);
 
 /* ---- partitioning ------------------------------------------------------ */
 

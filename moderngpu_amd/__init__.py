@@ -10,7 +10,7 @@ from .ops import (  # noqa: F401
     OPS, segreduce, transform_segreduce_mod13, spmv, load_balance_search,
     transform_lbs, interval_expand, interval_gather, interval_scatter,
     interval_move, load_balance_partitions, merge_path_partitions,
-    binary_search_partitions, segreduce_tile_size, lbs_tile_size, MgpuError,
+    binary_search_partitions, segreduce_tile_size, lbs_tile_size, lbs_search_tile_size, MgpuError,
     scan, reduce, lbs_segreduce_seg_plus_rank, workcreate,
     sorted_search, inner_join, prepare_segreduce, prepare_load_balance_search,
 )

@@ -14,6 +14,7 @@ SIGNATURES = {
     "mgpu_hip_error_string": (ctypes.c_char_p, [c_int]),
     "mgpu_hip_segreduce_tile_size": (c_int, [c_int]),
     "mgpu_hip_lbs_tile_size": (c_int, []),
+    "mgpu_hip_lbs_search_tile_size": (c_int, []),
     "mgpu_hip_partition_count": (c_int, [c_i64, c_i64, c_i64]),
     "mgpu_hip_load_balance_partitions": (c_int, [c_i64, c_vp, c_int, c_int, c_vp, c_vp]),
     "mgpu_hip_merge_path_partitions": (c_int, [c_vp, c_i64, c_vp, c_i64, c_i64, c_int, c_vp, c_vp]),

@@ -7,7 +7,14 @@ using namespace mgpu_hip;
 
 namespace {
 
+// Tiles of the kernels with cached values (expand, gather, scatter, move);
+// the workspace is sized for these, the smaller ones.  Kernels without cached
+// values (the search itself) use larger tiles and so fewer splits.
 typedef detail::lbs_launch_default_t lbs_launch_t;
+typedef detail::lbs_launch_plain_t lbs_plain_launch_t;
+static_assert(lbs_plain_launch_t::sm_ptx::nt * lbs_plain_launch_t::sm_ptx::vt >=
+  lbs_launch_t::sm_ptx::nt * lbs_launch_t::sm_ptx::vt,
+  "the workspace is sized for the smaller tile");
 
 // Plain byte bags for bit-for-bit element copies.
 struct alignas(16) bytes16_t { uint64_t lo, hi; };
@@ -126,8 +133,9 @@ int mgpu_hip_load_balance_search_phases(int count, const int* segments,
     (count && !output))
     return (int)hipErrorInvalidValue;
   return guarded(stream, [&](context_t& context) {
-    detail::transform_lbs_launch<lbs_launch_t>(store_seg_f { output }, count,
-      segments, num_segments, tuple<>(), (int*)workspace, phases, context);
+    detail::transform_lbs_launch<lbs_plain_launch_t>(store_seg_f { output },
+      count, segments, num_segments, tuple<>(), (int*)workspace, phases,
+      context);
   });
 }
 
@@ -144,7 +152,7 @@ int mgpu_hip_transform_lbs(int count, const int* segments, int num_segments,
   if(!lbs_args_ok(count, segments, num_segments, workspace, workspace_bytes))
     return (int)hipErrorInvalidValue;
   return guarded(stream, [&](context_t& context) {
-    detail::transform_lbs_launch<lbs_launch_t>(
+    detail::transform_lbs_launch<lbs_plain_launch_t>(
       store_seg_rank_f { seg_out, rank_out }, count, segments, num_segments,
       tuple<>(), (int*)workspace, detail::lbs_phase_all, context);
   });

@@ -66,6 +66,11 @@ int mgpu_hip_lbs_tile_size(void) {
     detail::lbs_launch_default_t::sm_ptx::vt);
 }
 
+int mgpu_hip_lbs_search_tile_size(void) {
+  return detail::lbs_tile_spacing(detail::lbs_launch_plain_t::sm_ptx::nt *
+    detail::lbs_launch_plain_t::sm_ptx::vt);
+}
+
 int mgpu_hip_partition_count(int64_t a_count, int64_t b_count,
   int64_t spacing) {
   if(a_count < 0 || b_count < 0 || spacing <= 0) return 0;

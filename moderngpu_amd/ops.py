@@ -73,6 +73,10 @@ def lbs_tile_size():
     return lib().mgpu_hip_lbs_tile_size()
 
 
+def lbs_search_tile_size():
+    return lib().mgpu_hip_lbs_search_tile_size()
+
+
 def _dtype_code(t, unsigned):
     if unsigned:
         want, code = _UNSIGNED["u32" if t.dtype == torch.int32 else "u64"]

@@ -33,6 +33,8 @@ def test_version_and_tile_sizes():
     assert m.segreduce_tile_size(5) % 64 == 0 and m.segreduce_tile_size(5) > 0
     assert m.segreduce_tile_size(99) == 0
     assert m.lbs_tile_size() % 64 == 0
+    assert m.lbs_search_tile_size() % 64 == 0
+    assert m.lbs_search_tile_size() >= m.lbs_tile_size()     # the workspace is sized for the smaller
 
 
 def test_partition_count_formula():

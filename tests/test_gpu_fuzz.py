@@ -10,7 +10,8 @@ import torch
 pytestmark = pytest.mark.gpu
 
 SIZES = [0, 1, 2, 63, 64, 65, 255, 256, 257, 2047, 2048, 2049, 4095, 4096, 4097,
-         6079, 6080, 6081, 6143, 6144, 6145, 8191, 8192, 12287, 12288, 20000, 50001]
+         6079, 6080, 6081, 6143, 6144, 6145, 8127, 8128, 8129, 8191, 8192, 12287, 12288,
+         16255, 16256, 16257, 20000, 50001]
 
 
 def _case(rng):

@@ -59,7 +59,9 @@ def test_lbs_reference_test_vector(dev):
 def test_lbs_layouts(dev, oracle):
     import moderngpu_amd as m
     rng = np.random.default_rng(13)
-    for name, count, segs in segment_layouts(rng, m.lbs_tile_size()):
+    layouts = list(segment_layouts(rng, m.lbs_search_tile_size())) + \
+        list(segment_layouts(rng, m.lbs_tile_size()))
+    for name, count, segs in layouts:
         got = m.load_balance_search(count, _dev(segs)).cpu().numpy()
         want = oracle.load_balance_search(count, segs)
         assert np.array_equal(got, want), name
