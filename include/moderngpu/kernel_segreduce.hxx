@@ -796,7 +796,6 @@ void spmv(matrix_it matrix, columns_it columns, vector_it vector,
   int count, segments_it segments, int num_segments, output_it output,
   context_t& context) {
 
-  typedef typename std::iterator_traits<matrix_it>::value_type type_t;
   detail::spmv_dispatch(matrix, columns, vector, count, segments,
     num_segments, output, context, launch_arg_t());
 }
