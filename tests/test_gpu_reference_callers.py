@@ -1,11 +1,11 @@
 """Runs the reference's own test programs (tests/test_load_balance.cu:1-34,
 test_sortedsearch.cu:1-33, test_reduce.cu:1-47, test_segreduce.cu:1-79,
-test_join.cu:1-10, test_intervalexpand.cu:1-9), compiled without any change
-against this library's headers: tests/csrc/Makefile builds them from where the
-reference tree lies into tests/csrc/reference_callers/ (binaries only; no
-source is copied).  Each program checks the device results against a host loop
-of its own.  test_scan.cu and test_intervalmove.cu are not built: they call
-the CUDA runtime by name.
+test_join.cu:1-10, test_intervalexpand.cu:1-9) and breadth-first-search demos,
+compiled without any change against this library's headers: oracle/Makefile
+builds them from where the reference tree lies into oracle/_ref/ (binaries
+only; no source is copied).  Each program checks the device results against a
+host loop of its own.  test_scan.cu and test_intervalmove.cu are not built:
+they call the CUDA runtime by name.
 
 The binaries exist only where they were built beside the reference tree; a
 checkout without them skips these tests."""
@@ -20,15 +20,15 @@ import numpy as np
 import pytest
 
 pytestmark = pytest.mark.gpu
-BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc",
-                   "reference_callers")
+BIN = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
+                   "oracle", "_ref")
 
 
 def _run(name, limit=110):
     """Returns (exit status, stdout, stderr)."""
     path = os.path.join(BIN, name)
     if not os.path.exists(path):
-        pytest.skip("reference_callers/%s was not built (no reference tree at build time)" % name)
+        pytest.skip("oracle/_ref/%s was not built (no reference tree at build time)" % name)
     proc = subprocess.run([path], capture_output=True, text=True, timeout=limit)
     return proc.returncode, proc.stdout, proc.stderr
 
@@ -38,7 +38,7 @@ def _run_for_a_while(name, seconds):
     line), ends it after `seconds` and returns (exit status or None, output)."""
     path = os.path.join(BIN, name)
     if not os.path.exists(path):
-        pytest.skip("reference_callers/%s was not built (no reference tree at build time)" % name)
+        pytest.skip("oracle/_ref/%s was not built (no reference tree at build time)" % name)
     master, slave = pty.openpty()
     proc = subprocess.Popen([path], stdout=slave, stderr=slave, stdin=subprocess.DEVNULL)
     os.close(slave)
@@ -161,7 +161,7 @@ def _bfs_levels(starts, dst, source):
 def _run_demo(name, tmp_path):
     path = os.path.join(BIN, name)
     if not os.path.exists(path):
-        pytest.skip("reference_callers/%s was not built (no reference tree at build time)" % name)
+        pytest.skip("oracle/_ref/%s was not built (no reference tree at build time)" % name)
     proc = subprocess.run([path], capture_output=True, text=True, timeout=110,
                           cwd=str(tmp_path))
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
