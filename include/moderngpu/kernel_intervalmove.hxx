@@ -123,6 +123,8 @@ template<typename launch_arg_t = empty_t, typename input_it,
   typename segments_it, typename output_it>
 void interval_expand(input_it input, int count, segments_it segments,
   int num_segments, output_it output, context_t& context) {
+  if(detail::launcher_interval<launch_arg_t>(input, count, segments,
+    num_segments, empty_t(), empty_t(), output, context)) return;
   typedef typename std::iterator_traits<input_it>::value_type type_t;
   detail::interval_expand_f<type_t, output_it> fill { output };
   transform_lbs<launch_arg_t>(fill, count, segments, num_segments,
@@ -135,6 +137,8 @@ template<typename launch_arg_t = empty_t, typename input_it,
   typename segments_it, typename gather_it, typename output_it>
 void interval_gather(input_it input, int count, segments_it segments,
   int num_segments, gather_it gather, output_it output, context_t& context) {
+  if(detail::launcher_interval<launch_arg_t>(input, count, segments,
+    num_segments, empty_t(), gather, output, context)) return;
   typename detail::interval_copy_select_t<false, true, input_it,
     output_it>::type copy { input, output };
   transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
@@ -148,6 +152,8 @@ template<typename launch_arg_t = empty_t, typename input_it,
 void interval_scatter(input_it input, int count, segments_it segments,
   int num_segments, scatter_it scatter, output_it output,
   context_t& context) {
+  if(detail::launcher_interval<launch_arg_t>(input, count, segments,
+    num_segments, scatter, empty_t(), output, context)) return;
   typename detail::interval_copy_select_t<true, false, input_it,
     output_it>::type copy { input, output };
   transform_lbs<launch_arg_t>(copy, count, segments, num_segments,
@@ -161,6 +167,8 @@ template<typename launch_arg_t = empty_t,
 void interval_move(input_it input, int count, segments_it segments,
   int num_segments, scatter_it scatter, gather_it gather, output_it output,
   context_t& context) {
+  if(detail::launcher_interval<launch_arg_t>(input, count, segments,
+    num_segments, scatter, gather, output, context)) return;
   typename detail::interval_copy_select_t<true, true, input_it,
     output_it>::type copy { input, output };
   transform_lbs<launch_arg_t>(copy, count, segments, num_segments,

@@ -12,6 +12,7 @@
 #pragma once
 #include "cta_load_balance.hxx"
 #include "search.hxx"
+#include "launcher.hxx"
 
 BEGIN_MGPU_NAMESPACE
 
@@ -309,6 +310,8 @@ template<typename launch_arg_t = empty_t, typename segments_it,
   typename output_it>
 void load_balance_search(int count, segments_it segments,
   int num_segments, output_it output, context_t& context) {
+  if(detail::launcher_load_balance_search<launch_arg_t>(count, segments,
+    num_segments, output, context)) return;
   transform_lbs<launch_arg_t>(detail::lbs_store_seg_f<output_it> { output },
     count, segments, num_segments, tuple<>(), context);
 }

@@ -36,6 +36,7 @@
 #include "cta_load_balance.hxx"
 #include "cta_segscan.hxx"
 #include "cta_segreduce.hxx"
+#include "launcher.hxx"
 #include "cta_reduce.hxx"
 #include "transform.hxx"
 #include "memory.hxx"
@@ -716,6 +717,9 @@ void segreduce(input_it input, int count, segments_it segments,
   int num_segments, output_it output, op_t op, type_t init,
   context_t& context) {
 
+  if(detail::launcher_segreduce<launch_arg_t>(input, count, segments,
+    num_segments, output, op, init, context)) return;
+
   typedef typename conditional_typedef_t<launch_arg_t,
     typename detail::segreduce_launch_default_t<type_t>::type_t_
   >::type_t launch_t;
@@ -796,6 +800,8 @@ void spmv(matrix_it matrix, columns_it columns, vector_it vector,
   int count, segments_it segments, int num_segments, output_it output,
   context_t& context) {
 
+  if(detail::launcher_spmv<launch_arg_t>(matrix, columns, vector, count,
+    segments, num_segments, output, context)) return;
   detail::spmv_dispatch(matrix, columns, vector, count, segments,
     num_segments, output, context, launch_arg_t());
 }

@@ -61,3 +61,7 @@ def test_runtime_helpers(dev):
 
 def test_caller_built_segreduce_from_cta_blocks(dev):
     assert "all passed" in _run("test_cta_segreduce")
+
+
+def test_templates_dispatch_to_the_prebuilt_library(dev):
+    assert "all passed" in _run("test_launcher")

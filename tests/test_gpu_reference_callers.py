@@ -70,9 +70,12 @@ def _run_for_a_while(name, seconds):
     return code, b"".join(chunks).decode(errors="replace")
 
 
-def test_reference_test_load_balance(dev):
+@pytest.mark.parametrize("name", ["test_load_balance", "launcher_test_load_balance"])
+def test_reference_test_load_balance(dev, name):
     # Prints one line per item of 200,030 and "ERROR AT" (then exit(0)) on a mismatch.
-    code, out, err = _run("test_load_balance")
+    # The launcher_ build defines MGPU_HIP_LAUNCHER: its load_balance_search
+    # runs the prebuilt kernels of libmgpu_hip.so.
+    code, out, err = _run(name)
     assert code == 0, err[-2000:]
     assert "ERROR" not in out
     lines = re.findall(r"^ *(\d+): +(\d+)$", out, flags=re.M)
