@@ -95,6 +95,8 @@ template<typename launch_arg_t = empty_t, typename input_it,
 void reduce(input_it input, int count, output_it reduction, op_t op,
   context_t& context) {
 
+  if(detail::launcher_reduce<launch_arg_t>(input, count, reduction, op,
+    context)) return;
   typedef typename std::iterator_traits<input_it>::value_type type_t;
   typedef typename conditional_typedef_t<launch_arg_t,
     typename detail::scan_launch_default_t<type_t>::type_t_>::type_t launch_t;

@@ -23,6 +23,7 @@
 #include "memory.hxx"
 #include "operators.hxx"
 #include "transform.hxx"
+#include "launcher.hxx"
 
 BEGIN_MGPU_NAMESPACE
 
@@ -323,6 +324,8 @@ template<scan_type_t scan_type = scan_type_exc,
 void scan_event(input_it input, int count, output_it output, op_t op,
   reduction_it reduction, context_t& context, hipEvent_t event) {
 
+  if(detail::launcher_scan<launch_arg_t>(scan_type_inc == scan_type, input,
+    count, output, op, reduction, context, event)) return;
   typedef typename std::iterator_traits<input_it>::value_type type_t;
   typedef typename conditional_typedef_t<launch_arg_t,
     typename detail::scan_launch_default_t<type_t>::type_t_>::type_t launch_t;

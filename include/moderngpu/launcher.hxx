@@ -7,8 +7,8 @@
 // including these headers and links libmgpu_hip.so gets, for the argument
 // combinations the extern "C" layer covers -- raw pointers, value types
 // {int, unsigned, 64-bit ints, float, double}, operators plus_t / maximum_t /
-// minimum_t, element sizes 1/2/4/8/16 bytes for the interval functions, no
-// explicit launch box -- a call into that layer instead: the same kernels,
+// minimum_t (segreduce, scan, reduce; spmv on float / double), element sizes
+// 1/2/4/8/16 bytes for the interval functions, no explicit launch box -- a call into that layer instead: the same kernels,
 // compiled once, and nothing of them in the caller's object code.  Everything
 // else (functors, iterators, user types and operators, explicit launch boxes)
 // still instantiates in place.  Temporaries come from context.alloc() and the
@@ -201,6 +201,59 @@ bool launcher_interval(input_it input, int count,
     return false;
 }
 
+// scan / scan_event without an event; the fold goes to a type_t* or is
+// discarded.
+template<typename launch_arg_t, typename input_it, typename output_it,
+  typename op_t, typename reduction_it>
+bool launcher_scan(bool inclusive, input_it input, int count,
+  output_it output, op_t, reduction_it reduction, context_t& context,
+  hipEvent_t event) {
+  typedef typename std::iterator_traits<input_it>::value_type type_t;
+  enum { discards =
+    std::is_same<reduction_it, discard_iterator_t<type_t> >::value };
+  if constexpr(std::is_same<launch_arg_t, empty_t>::value &&
+    launcher_dtype_t<type_t>::value >= 0 &&
+    launcher_op_t<op_t, type_t>::value >= 0 &&
+    launcher_points_to_t<input_it, type_t>::value &&
+    launcher_points_to_t<output_it, type_t, true>::value &&
+    (discards || launcher_points_to_t<reduction_it, type_t, true>::value)) {
+    if(event) return false;         // the layer cannot record one mid-call
+    int dtype = launcher_dtype_t<type_t>::value;
+    size_t bytes = mgpu_hip_scan_workspace_bytes(count, dtype);
+    mem_t<char> workspace(bytes, context);
+    void* total = nullptr;
+    if constexpr(!discards) total = reduction;
+    launcher_check(mgpu_hip_scan(input, count, output, dtype,
+      launcher_op_t<op_t, type_t>::value, (int)inclusive, total,
+      workspace.data(), bytes, context.stream()));
+    ++launcher_calls();
+    return true;
+  } else
+    return false;
+}
+
+template<typename launch_arg_t, typename input_it, typename output_it,
+  typename op_t>
+bool launcher_reduce(input_it input, int count, output_it reduction, op_t,
+  context_t& context) {
+  typedef typename std::iterator_traits<input_it>::value_type type_t;
+  if constexpr(std::is_same<launch_arg_t, empty_t>::value &&
+    launcher_dtype_t<type_t>::value >= 0 &&
+    launcher_op_t<op_t, type_t>::value >= 0 &&
+    launcher_points_to_t<input_it, type_t>::value &&
+    launcher_points_to_t<output_it, type_t, true>::value) {
+    int dtype = launcher_dtype_t<type_t>::value;
+    size_t bytes = mgpu_hip_reduce_workspace_bytes(count, dtype);
+    mem_t<char> workspace(bytes, context);
+    launcher_check(mgpu_hip_reduce(input, count, reduction, dtype,
+      launcher_op_t<op_t, type_t>::value, workspace.data(), bytes,
+      context.stream()));
+    ++launcher_calls();
+    return true;
+  } else
+    return false;
+}
+
 #else // !MGPU_HIP_LAUNCHER
 
 template<typename launch_arg_t, typename... args_t>
@@ -213,6 +266,10 @@ constexpr bool launcher_load_balance_search(const args_t&...) {
 }
 template<typename launch_arg_t, typename... args_t>
 constexpr bool launcher_interval(const args_t&...) { return false; }
+template<typename launch_arg_t, typename... args_t>
+constexpr bool launcher_scan(const args_t&...) { return false; }
+template<typename launch_arg_t, typename... args_t>
+constexpr bool launcher_reduce(const args_t&...) { return false; }
 
 #endif
 

@@ -8,6 +8,7 @@
 #endif
 #include <moderngpu/kernel_segreduce.hxx>
 #include <moderngpu/kernel_intervalmove.hxx>
+#include <moderngpu/kernel_reduce.hxx>
 #include <algorithm>
 #include <climits>
 #include <cstdio>
@@ -202,6 +203,43 @@ int main() {
       for(int i = segs[seg]; i < e; ++i) { want += (double)a[i] * x[c[i]]; norm += (double)a[i] * x[c[i]]; }
       CHECK(std::abs(got[seg] - want) <= 1e-5 * norm + 1e-30);
     }
+  }
+  {
+    // scan and reduce on pointers -> library (not when an event is to be
+    // recorded mid-call, and not for computed inputs).
+    int n = 1 << 20;
+    std::vector<int> hv(n);
+    std::mt19937 mt(17);
+    for(int& x : hv) x = (int)(mt() % 200) - 100;
+    mem_t<int> v = to_mem(hv, context), scanned(n, context), total(1, context);
+    calls = detail::launcher_calls();
+    scan((const int*)v.data(), n, scanned.data(), plus_t<int>(), total.data(), context);
+    CHECK(detail::launcher_calls() == calls + 1);
+    std::vector<int> got = from_mem(scanned);
+    int run = 0;
+    for(int i = 0; i < n; ++i) { CHECK(got[i] == run); run += hv[i]; }
+    CHECK(from_mem(total)[0] == run);
+
+    scan<scan_type_inc>(v.data(), n, scanned.data(), maximum_t<int>(),
+      discard_iterator_t<int>(), context);
+    CHECK(detail::launcher_calls() == calls + 2);
+    got = from_mem(scanned);
+    int best = hv[0];
+    for(int i = 0; i < n; ++i) { best = std::max(best, hv[i]); CHECK(got[i] == best); }
+
+    reduce((const int*)v.data(), n, total.data(), plus_t<int>(), context);
+    CHECK(detail::launcher_calls() == calls + 3);
+    CHECK(from_mem(total)[0] == run);
+
+    hipEvent_t event;
+    CHECK(hipSuccess == hipEventCreate(&event));
+    scan_event(v.data(), n, scanned.data(), plus_t<int>(), total.data(), context, event);
+    const int* data = v.data();
+    transform_reduce([=]MGPU_DEVICE(int i) { return data[i]; }, n, total.data(),
+      plus_t<int>(), context);
+    CHECK(detail::launcher_calls() == calls + 3);
+    CHECK(from_mem(total)[0] == run);
+    CHECK(hipSuccess == hipEventDestroy(event));
   }
   {
     // An error from the layer comes back as the library's exception.
