@@ -100,3 +100,52 @@ def test_search_and_join_fuzz(oracle, dev, seed):
         if n * h < 4_000_000 or hi > 100:
             got = m.inner_join(da, db)
             assert np.array_equal(got.cpu().numpy(), oracle.inner_join(a, b)), (seed, n, h, hi)
+
+
+def test_large_random_shapes(oracle, dev):
+    """Hundreds of tiles per call: counts up to 2 * 10^6 with few, many, far too
+    many and Zipf-distributed segments, for the search (both outputs), interval
+    expand on 4- and 8-byte values and an int32 segmented sum."""
+    import moderngpu_amd as m
+    rng = np.random.default_rng(77)
+    for case in range(60):
+        count = int(rng.integers(0, 2_000_000))
+        kind = case % 5
+        if kind == 0:
+            nseg = int(rng.integers(1, 50))
+        elif kind == 1:
+            nseg = max(1, count // int(rng.integers(1, 64)))
+        elif kind == 2:
+            nseg = int(rng.integers(1, 3_000_000))
+        elif kind == 3:
+            nseg = max(1, count // 3)
+        else:
+            nseg = int(rng.integers(1, 20000))
+        starts = np.zeros(nseg, dtype=np.int32)
+        if nseg > 1:
+            if case % 7 == 0:
+                lens = np.minimum(rng.zipf(1.3, size=nseg), 1 << 16).astype(np.int64)
+                lens = (lens * (count / max(1, lens.sum()))).astype(np.int64)
+                starts[1:] = np.minimum(np.cumsum(lens)[:-1], count)
+            else:
+                starts[1:] = np.sort(rng.integers(0, count + 1, size=nseg - 1))
+        tag = (case, count, nseg)
+        segs = torch.from_numpy(starts).to(dev)
+        want = oracle.load_balance_search(count, starts)
+        got = m.load_balance_search(count, segs).cpu().numpy()
+        assert np.array_equal(got, want), ("lbs",) + tag
+        seg, rank = m.transform_lbs(count, segs)
+        assert np.array_equal(seg.cpu().numpy(), want), ("transform_lbs seg",) + tag
+        assert np.array_equal(rank.cpu().numpy(),
+                              np.arange(count, dtype=np.int64) - starts[want]), \
+            ("transform_lbs rank",) + tag
+        for dtype, top in ((np.int32, 1 << 30), (np.int64, 1 << 60)):
+            per_seg = rng.integers(0, top, size=nseg).astype(dtype)
+            got = m.interval_expand(torch.from_numpy(per_seg).to(dev), count, segs)
+            assert np.array_equal(got.cpu().numpy(),
+                                  oracle.interval_expand(per_seg, count, starts)), \
+                ("expand", dtype.__name__) + tag
+        vals = rng.integers(-1000, 1000, size=count).astype(np.int32)
+        got = m.segreduce(torch.from_numpy(vals).to(dev), segs, "plus", -5)
+        assert np.array_equal(got.cpu().numpy(),
+                              oracle.segreduce(vals, starts, "plus", -5)), ("segreduce",) + tag
