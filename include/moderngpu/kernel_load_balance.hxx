@@ -122,75 +122,76 @@ struct transform_lbs_f {
 
     PRAGMA_UNROLL
     for(int g = 0; g < tiles_per_cta; ++g) {
-    if(tiles_per_cta * group + g >= num_tiles) break;
-    if(g) __syncthreads();            // the previous tile is done with LDS
+      if(tiles_per_cta * group + g >= num_tiles) break;
+      if(g) __syncthreads();            // the previous tile is done with LDS
 
-    // After fill(), LDS slot p holds (segment of tile item p) - seg_base and
-    // the tile's segment starts sit behind the slots.
-    merge_range_t range = ranges[g];
-    int a_count = range.a_count();
-    int seg_base = range.b_begin - 1;
-    load_balance_t().fill(range, segments, tid, shared.lbs, ahead[g]);
-    cached_load_t::commit(tid, seg_base, range.b_count() + 1, fetched[g],
-      shared.cached);
-    const int* slots = shared.lbs.indices;
-    const int* starts = slots + load_balance_t::starts_offset(a_count);
+      // After fill(), LDS slot p holds (segment of tile item p) - seg_base and
+      // the tile's segment starts sit behind the slots.
+      merge_range_t range = ranges[g];
+      int a_count = range.a_count();
+      int seg_base = range.b_begin - 1;
+      load_balance_t().fill(range, segments, tid, shared.lbs, ahead[g]);
+      cached_load_t::commit(tid, seg_base, range.b_count() + 1, fetched[g],
+        shared.cached);
+      const int* slots = shared.lbs.indices;
+      const int* starts = slots + load_balance_t::starts_offset(a_count);
 
-    // The emission loop exists twice -- cached values staged in LDS, or
-    // gathered from global memory -- so that each copy is straight-line code.
-    auto emit_all = [&](auto staged_tag) {
-      if constexpr(is_chunk_functor_t<func_t>::value) {
-        // The functor consumes W consecutive items at a time (one 16-byte
-        // store per chunk for 4-byte results).  Chunk nt * i + tid in step i:
-        // consecutive lanes own consecutive chunks.
-        PRAGMA_UNROLL
-        for(int i = 0; i < chunks; ++i) {
-          int p = W * (nt * i + tid);
-          int index = range.a_begin + p;
-          if(p + W <= a_count) {
-            int rel[W], seg[W], rank[W];
-            value_t cached[W];
-            lds_load_chunk<W>(slots + layout_t::index(p), rel);
-            PRAGMA_UNROLL
-            for(int e = 0; e < W; ++e) {
-              seg[e] = seg_base + rel[e];
-              rank[e] = index + e - starts[rel[e]];
-              cached[e] = cached_load_t::get(decltype(staged_tag)::value, rel[e], seg[e],
-                shared.cached, caching_iterators);
-            }
-            f.template chunk<W>(index, seg, rank, cached, args...);
-          } else {
-            PRAGMA_UNROLL
-            for(int e = 0; e < W; ++e) {
-              if(p + e < a_count) {
-                int rel = slots[layout_t::index(p + e)];
-                int seg = seg_base + rel;
-                f(index + e, seg, index + e - starts[rel],
-                  cached_load_t::get(decltype(staged_tag)::value, rel, seg, shared.cached,
-                    caching_iterators), args...);
+      // The emission loop exists twice -- cached values staged in LDS, or
+      // gathered from global memory -- so that each copy is straight-line code.
+      auto emit_all = [&](auto staged_tag) {
+        constexpr bool in_lds = decltype(staged_tag)::value;
+        if constexpr(is_chunk_functor_t<func_t>::value) {
+          // The functor consumes W consecutive items at a time (one 16-byte
+          // store per chunk for 4-byte results).  Chunk nt * i + tid in step i:
+          // consecutive lanes own consecutive chunks.
+          PRAGMA_UNROLL
+          for(int i = 0; i < chunks; ++i) {
+            int p = W * (nt * i + tid);
+            int index = range.a_begin + p;
+            if(p + W <= a_count) {
+              int rel[W], seg[W], rank[W];
+              value_t cached[W];
+              lds_load_chunk<W>(slots + layout_t::index(p), rel);
+              PRAGMA_UNROLL
+              for(int e = 0; e < W; ++e) {
+                seg[e] = seg_base + rel[e];
+                rank[e] = index + e - starts[rel[e]];
+                cached[e] = cached_load_t::get(in_lds, rel[e], seg[e],
+                  shared.cached, caching_iterators);
+              }
+              f.template chunk<W>(index, seg, rank, cached, args...);
+            } else {
+              PRAGMA_UNROLL
+              for(int e = 0; e < W; ++e) {
+                if(p + e < a_count) {
+                  int rel = slots[layout_t::index(p + e)];
+                  int seg = seg_base + rel;
+                  f(index + e, seg, index + e - starts[rel],
+                    cached_load_t::get(in_lds, rel, seg, shared.cached,
+                      caching_iterators), args...);
+                }
               }
             }
           }
-        }
-      } else {
-        // One item per call, item nt * i + tid in step i: whatever the functor
-        // stores per item is coalesced across the wavefront.
-        PRAGMA_UNROLL
-        for(int i = 0; i < vt; ++i) {
-          int p = nt * i + tid;
-          if(p < a_count) {
-            int rel = slots[layout_t::index(p)];
-            int seg = seg_base + rel;
-            int index = range.a_begin + p;
-            f(index, seg, index - starts[rel],
-              cached_load_t::get(decltype(staged_tag)::value, rel, seg, shared.cached,
-                caching_iterators), args...);
+        } else {
+          // One item per call, item nt * i + tid in step i: whatever the
+          // functor stores per item is coalesced across the wavefront.
+          PRAGMA_UNROLL
+          for(int i = 0; i < vt; ++i) {
+            int p = nt * i + tid;
+            if(p < a_count) {
+              int rel = slots[layout_t::index(p)];
+              int seg = seg_base + rel;
+              int index = range.a_begin + p;
+              f(index, seg, index - starts[rel],
+                cached_load_t::get(in_lds, rel, seg, shared.cached,
+                  caching_iterators), args...);
+            }
           }
         }
-      }
-    };
-    if(staged[g]) emit_all(std::true_type());
-    else emit_all(std::false_type());
+      };
+      if(staged[g]) emit_all(std::true_type());
+      else emit_all(std::false_type());
     }
   }
 };

@@ -8,7 +8,8 @@
 //
 // Two launches: one partial per tile (the scan's upsweep kernel: 16-byte
 // strided loads, thread order through LDS), then one CTA folds the partials
-// the same way.  Inputs of a few thousand items go to that CTA directly.  Interface after src/moderngpu/kernel_reduce.hxx:11-68.
+// the same way.  Inputs of a few thousand items go to that CTA directly.
+// Interface after src/moderngpu/kernel_reduce.hxx:11-68.
 #pragma once
 #include "kernel_scan.hxx"
 

@@ -8,8 +8,9 @@
 // combinations the extern "C" layer covers -- raw pointers, value types
 // {int, unsigned, 64-bit ints, float, double}, operators plus_t / maximum_t /
 // minimum_t (segreduce, scan, reduce; spmv on float / double), element sizes
-// 1/2/4/8/16 bytes for the interval functions, no explicit launch box -- a call into that layer instead: the same kernels,
-// compiled once, and nothing of them in the caller's object code.  Everything
+// 1/2/4/8/16 bytes for the interval functions, no explicit launch box -- a
+// call into that layer instead: the same kernels, compiled once, and nothing
+// of them in the caller's object code.  Everything
 // else (functors, iterators, user types and operators, explicit launch boxes)
 // still instantiates in place.  Temporaries come from context.alloc() and the
 // launches go to context.stream(), as in the header-only path; a non-zero
@@ -76,7 +77,7 @@ struct launcher_elem_bytes_t {
     size = (int)sizeof(type_t),
     value = std::is_trivially_copyable<type_t>::value &&
       (1 == size || 2 == size || 4 == size || 8 == size || 16 == size) &&
-      (int)alignof(type_t) >= size      // the layer moves naturally aligned words
+      (int)alignof(type_t) >= size    // the layer moves naturally aligned words
   };
 };
 
