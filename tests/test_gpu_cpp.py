@@ -65,3 +65,9 @@ def test_caller_built_segreduce_from_cta_blocks(dev):
 
 def test_templates_dispatch_to_the_prebuilt_library(dev):
     assert "all passed" in _run("test_launcher")
+
+
+def test_nearest_cities_pipeline_on_the_reference_demo_data(dev):
+    sample = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden",
+                          "statecity_sample.csv")
+    assert "all passed" in _run("test_cities", sample)
