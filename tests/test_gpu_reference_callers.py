@@ -189,3 +189,34 @@ def test_reference_demo_bfs3_fronts(dev, tmp_path):
     got = [(int(v), int(e)) for v, e in re.findall(
         r"Front for level \d+ has (\d+) vertices and (\d+) edges", out)]
     assert got == fronts
+
+
+# ---- the tutorials on the launch mechanism (tutorial/tut_01_transform.cu,
+# tut_02_cta_launch.cu, tut_03_launch_box.cu, tut_04_launch_custom.cu) --------
+
+def test_reference_tutorial_transform(dev):
+    # Ten device threads print a line each.
+    code, out, err = _run("tut_01_transform")
+    assert code == 0, err[-2000:]
+    threads = sorted(int(n) for n in re.findall(r"Thread (\d+) says the year is \d{4}", out))
+    assert threads == list(range(10))
+
+
+def test_reference_tutorial_cta_launch(dev):
+    # A 16-thread CTA sums the first 16 squares through LDS.
+    code, out, err = _run("tut_02_cta_launch")
+    assert code == 0, err[-2000:]
+    assert "Reduction of 16 elements is %d" % sum(i * i for i in range(1, 17)) in out
+
+
+def test_reference_tutorial_launch_boxes(dev):
+    # A box written for CUDA architectures resolves the way the reference
+    # resolves it for its newest architecture (launch_box.hxx:31-45: sm_86 ->
+    # 80 -> 75 -> 70 -> 62 -> 60 -> 53 -> 50 -> 35 -> 30 -> 21 -> 20, which
+    # passes sm_52 by): tut_03's box to its sm_50 entry, tut_04's to sm_35.
+    code, out, err = _run("tut_03_launch_box")
+    assert code == 0, err[-2000:]
+    assert "Standard launch box: nt = 256 vt = 8" in out
+    code, out, err = _run("tut_04_launch_custom")
+    assert code == 0, err[-2000:]
+    assert "Custom launch box: nt = 128 mode = 2000 sizeof(type_t)=4" in out
