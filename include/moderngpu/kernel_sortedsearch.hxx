@@ -17,6 +17,7 @@
 #pragma once
 #include "search.hxx"
 #include "cta_load_balance.hxx"
+#include "launcher.hxx"
 
 BEGIN_MGPU_NAMESPACE
 
@@ -147,6 +148,9 @@ void sorted_search(needles_it needles, int num_needles, haystack_it haystack,
   typedef typename conditional_typedef_t<launch_arg_t,
     detail::sorted_search_launch_default_t>::type_t launch_t;
   if(num_needles <= 0) return;
+  if(detail::launcher_sorted_search<launch_arg_t>(bounds_upper == bounds,
+    needles, num_needles, haystack, num_haystack, indices, comp, context))
+    return;
   int64_t total = (int64_t)num_needles + num_haystack;
   mem_t<int> partitions((size_t)div_up(total, (int64_t)launch_t::nv(context))
     + 1, context);

@@ -255,6 +255,42 @@ bool launcher_reduce(input_it input, int count, output_it reduction, op_t,
     return false;
 }
 
+// sorted_search on int keys ordered by less_t<int>.
+template<typename launch_arg_t, typename needles_it, typename haystack_it,
+  typename indices_it, typename comp_t>
+bool launcher_sorted_search(bool upper, needles_it needles, int num_needles,
+  haystack_it haystack, int num_haystack, indices_it indices, comp_t,
+  context_t& context) {
+  if constexpr(std::is_same<launch_arg_t, empty_t>::value &&
+    std::is_same<comp_t, less_t<int> >::value &&
+    launcher_points_to_t<needles_it, int>::value &&
+    launcher_points_to_t<haystack_it, int>::value &&
+    launcher_points_to_t<indices_it, int, true>::value) {
+    size_t bytes = mgpu_hip_sorted_search_workspace_bytes(num_needles,
+      num_haystack);
+    mem_t<char> workspace(bytes, context);
+    launcher_check(mgpu_hip_sorted_search(needles, num_needles, haystack,
+      num_haystack, upper ? MGPU_BOUNDS_UPPER : MGPU_BOUNDS_LOWER, indices,
+      workspace.data(), bytes, context.stream()));
+    ++launcher_calls();
+    return true;
+  } else
+    return false;
+}
+
+// load_balance_partitions into an int array.
+template<typename segments_it>
+bool launcher_load_balance_partitions(int64_t count, segments_it segments,
+  int num_segments, int spacing, int* partitions, context_t& context) {
+  if constexpr(launcher_points_to_t<segments_it, int>::value) {
+    launcher_check(mgpu_hip_load_balance_partitions(count, segments,
+      num_segments, spacing, partitions, context.stream()));
+    ++launcher_calls();
+    return true;
+  } else
+    return false;
+}
+
 #else // !MGPU_HIP_LAUNCHER
 
 template<typename launch_arg_t, typename... args_t>
@@ -271,6 +307,12 @@ template<typename launch_arg_t, typename... args_t>
 constexpr bool launcher_scan(const args_t&...) { return false; }
 template<typename launch_arg_t, typename... args_t>
 constexpr bool launcher_reduce(const args_t&...) { return false; }
+template<typename launch_arg_t, typename... args_t>
+constexpr bool launcher_sorted_search(const args_t&...) { return false; }
+template<typename... args_t>
+constexpr bool launcher_load_balance_partitions(const args_t&...) {
+  return false;
+}
 
 #endif
 

@@ -9,6 +9,7 @@
 #include "cta_search.hxx"
 #include "memory.hxx"
 #include "context.hxx"
+#include "launcher.hxx"
 
 BEGIN_MGPU_NAMESPACE
 
@@ -364,6 +365,10 @@ auto load_balance_partitions(int64_t dest_count, segments_it segments,
   int num_partitions = (int)div_up(dest_count + num_segments,
     (int64_t)spacing) + 1;
   mem_t<int_t> mem(num_partitions, context);
+  if constexpr(std::is_same<int_t, int>::value) {
+    if(detail::launcher_load_balance_partitions(dest_count, segments,
+      num_segments, spacing, mem.data(), context)) return mem;
+  }
   load_balance_partitions_into(dest_count, segments, num_segments, spacing,
     mem.data(), context);
   return mem;

@@ -9,6 +9,7 @@
 #include <moderngpu/kernel_segreduce.hxx>
 #include <moderngpu/kernel_intervalmove.hxx>
 #include <moderngpu/kernel_reduce.hxx>
+#include <moderngpu/kernel_sortedsearch.hxx>
 #include <algorithm>
 #include <climits>
 #include <cstdio>
@@ -240,6 +241,36 @@ int main() {
     CHECK(detail::launcher_calls() == calls + 3);
     CHECK(from_mem(total)[0] == run);
     CHECK(hipSuccess == hipEventDestroy(event));
+  }
+  {
+    // sorted_search on int keys with less_t and load_balance_partitions.
+    int n = 200000, h = 150000;
+    mem_t<int> needles = fill_random(0, 1 << 20, n, true, context);
+    mem_t<int> hay = fill_random(0, 1 << 20, h, true, context);
+    mem_t<int> found(n, context);
+    calls = detail::launcher_calls();
+    sorted_search<bounds_upper>((const int*)needles.data(), n,
+      (const int*)hay.data(), h, found.data(), less_t<int>(), context);
+    CHECK(detail::launcher_calls() == calls + 1);
+    std::vector<int> hn = from_mem(needles), hh = from_mem(hay), got = from_mem(found);
+    for(int i = 0; i < n; ++i)
+      CHECK(got[i] == (int)(std::upper_bound(hh.begin(), hh.end(), hn[i]) - hh.begin()));
+    sorted_search<bounds_lower>(needles.data(), n, hay.data(), h, found.data(),
+      [=]MGPU_DEVICE(int a, int b) { return a < b; }, context);   // a lambda: stays here
+    CHECK(detail::launcher_calls() == calls + 1);
+    got = from_mem(found);
+    for(int i = 0; i < n; ++i)
+      CHECK(got[i] == (int)(std::lower_bound(hh.begin(), hh.end(), hn[i]) - hh.begin()));
+
+    mem_t<int> mp = load_balance_partitions(count, s.data(), num_segments, 1000, context);
+    CHECK(detail::launcher_calls() == calls + 2);
+    std::vector<int> hmp = from_mem(mp);
+    CHECK((int)hmp.size() == div_up(count + num_segments, 1000) + 1);
+    for(size_t i = 0; i < hmp.size(); ++i) {
+      int diag = std::min((int)(1000 * i), count + num_segments);
+      CHECK(hmp[i] == merge_path<bounds_upper>(counting_iterator_t<int>(0), count,
+        segs.data(), num_segments, diag, less_t<int>()));
+    }
   }
   {
     // An error from the layer comes back as the library's exception.
