@@ -8,6 +8,7 @@
 //    joins of random keys checked pair by pair against a host loop.
 // Exit status 1 on the first mismatch.
 #include <moderngpu/kernel_join.hxx>
+#include <moderngpu/kernel_merge.hxx>
 #include <algorithm>
 #include <cstdio>
 #include <functional>
@@ -196,8 +197,39 @@ static int check_cta_merge(int na, int nb, int max_key, context_t& context) {
   return 0;
 }
 
+// merge(): keys with values and keys alone, against a host merge.
+template<typename launch_t>
+static int check_merge(int na, int nb, int max_key, context_t& context) {
+  mem_t<int> a = fill_random(0, max_key, na, true, context);
+  mem_t<int> b = fill_random(0, max_key, nb, true, context);
+  mem_t<int> a_vals(na, context), b_vals(nb, context);
+  int* av = a_vals.data(); int* bv = b_vals.data();
+  transform([=]MGPU_DEVICE(int i) { av[i] = i; }, na, context);
+  transform([=]MGPU_DEVICE(int i) { bv[i] = -1 - i; }, nb, context);
+  mem_t<int> keys(na + nb, context), vals(na + nb, context), only(na + nb, context);
+  merge<launch_t>(a.data(), a_vals.data(), na, b.data(), b_vals.data(), nb,
+    keys.data(), vals.data(), less_t<int>(), context);
+  merge<launch_t>(a.data(), na, b.data(), nb, only.data(), less_t<int>(), context);
+  std::vector<int> ha = from_mem(a), hb = from_mem(b), hk = from_mem(keys),
+    hv = from_mem(vals), ho = from_mem(only);
+  int ia = 0, ib = 0;
+  for(int p = 0; p < na + nb; ++p) {
+    bool take_a = ia < na && (ib >= nb || !(hb[ib] < ha[ia]));
+    int key = take_a ? ha[ia] : hb[ib];
+    CHECK(hk[p] == key && ho[p] == key);
+    CHECK(hv[p] == (take_a ? ia : -1 - ib));
+    if(take_a) ++ia; else ++ib;
+  }
+  return 0;
+}
+
 int main() {
   standard_context_t context(false);
+  CHECK(0 == check_merge<empty_t>(1000000, 700000, 1 << 20, context));
+  CHECK(0 == check_merge<empty_t>(5000, 300000, 50, context));
+  CHECK(0 == (check_merge<launch_params_t<128, 7> >(100000, 99999, 1000, context)));
+  CHECK(0 == check_merge<empty_t>(0, 4096, 100, context));
+  CHECK(0 == check_merge<empty_t>(1, 0, 100, context));
   CHECK(0 == (check_cta_merge<128, 7>(100000, 130000, 5000, context)));
   CHECK(0 == (check_cta_merge<64, 4>(3000, 50, 40, context)));
   CHECK(0 == (check_cta_merge<256, 3>(1, 70000, 1 << 30, context)));

@@ -220,3 +220,20 @@ def test_reference_tutorial_launch_boxes(dev):
     code, out, err = _run("tut_04_launch_custom")
     assert code == 0, err[-2000:]
     assert "Custom launch box: nt = 128 mode = 2000 sizeof(type_t)=4" in out
+
+
+def test_reference_tutorial_iterators(dev):
+    # A computed sequence (Fibonacci numbers from a load iterator) is merged
+    # with a strided one into a store iterator that also takes logarithms.
+    import math
+    code, out, err = _run("tut_05_iterators")
+    assert code == 0, err[-2000:]
+    fib = [0, 1]
+    while len(fib) < 20:
+        fib.append(fib[-1] + fib[-2])
+    listed = {int(i): int(v) for i, v in re.findall(r"Fibonacci +(\d+) = +(\d+)", out)}
+    assert listed == dict(enumerate(fib))
+    merged = [(int(k), float(v)) for k, v in re.findall(r"log\( *(\d+)\) = ([-0-9.]+)", out)]
+    assert [k for k, _ in merged] == sorted(fib + [50 + 500 * i for i in range(10)])
+    for k, v in merged:
+        assert abs(v - (math.log(k) if k else 0.0)) < 1e-5
