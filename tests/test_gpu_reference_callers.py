@@ -1,6 +1,7 @@
 """Runs the reference's own test programs (tests/test_load_balance.cu:1-34,
 test_sortedsearch.cu:1-33, test_reduce.cu:1-47, test_segreduce.cu:1-79,
-test_join.cu:1-10, test_intervalexpand.cu:1-9) and breadth-first-search demos,
+test_join.cu:1-10, test_intervalexpand.cu:1-9, test_merge.cu:1-37), its
+breadth-first-search demos and its tutorials,
 compiled without any change against this library's headers: oracle/Makefile
 builds them from where the reference tree lies into oracle/_ref/ (binaries
 only; no source is copied).  Each program checks the device results against a
@@ -106,6 +107,16 @@ def test_reference_test_segreduce(dev):
     assert code in (None, 0), out[-2000:]
     assert "error" not in out.lower()
     assert out.count("passed") >= 3, out[-2000:]
+
+
+def test_reference_test_merge(dev):
+    # Sizes from 1,000 to 10^8 in steps of 10 %, each merged on the device and
+    # with std::merge (the inputs are sorted on the host, which takes most of
+    # the time at the large sizes); ended after a while like test_segreduce.
+    code, out = _run_for_a_while("test_merge", 25)
+    assert code in (None, 0), out[-2000:]
+    assert "FAILURE" not in out
+    assert out.count("SUCCESS") >= 60, out[-2000:]
 
 
 def test_reference_test_join_and_intervalexpand(dev):
