@@ -390,7 +390,11 @@ struct cta_load_balance_t {
       for(int r = 0; r < prefetch_rows; ++r)
         if(nt * r + tid < b_count)
           ahead.starts[r] = segments[range.b_begin + nt * r + tid];
-      if(!tid && range.b_begin) ahead.preceding = segments[range.b_begin - 1];
+      // The start in front of the tile's own is read by the last thread: a
+      // read by thread 0 alone becomes a scalar load that the first wavefront
+      // waits for on the spot.
+      if(nt - 1 == tid && range.b_begin)
+        ahead.preceding = segments[range.b_begin - 1];
     }
     return ahead;
   }
@@ -428,7 +432,7 @@ struct cta_load_balance_t {
       PRAGMA_UNROLL
       for(int r = 0; r < prefetch_rows; ++r)
         if(nt * r + tid < b_count) starts[1 + nt * r + tid] = ahead.starts[r];
-      if(!tid) starts[0] = ahead.preceding;
+      if(nt - 1 == tid) starts[0] = ahead.preceding;
     } else {
       for(int j = tid; j < b_count; j += nt)
         starts[1 + j] = segments[range.b_begin + j];
