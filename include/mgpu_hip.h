@@ -102,6 +102,27 @@ MGPU_HIP_API int mgpu_hip_segreduce(const void* input, int count,
   const void* init, void* workspace, size_t workspace_bytes,
   mgpu_stream_t stream);
 
+/* mgpu_hip_segreduce for callers that cannot allocate device memory (code
+ * under HIP graph capture, serving loops, harnesses that forbid hipMalloc).
+ * No counterpart in the reference, whose segreduce allocates its temporaries
+ * through the context on every call (kernel_segreduce.hxx:210-216).  Same
+ * arguments and results as mgpu_hip_segreduce without the workspace: the
+ * tile splits and per-tile carries live in a device array of
+ * MGPU_HIP_STATIC_SCRATCH_BYTES that the library holds on every GPU it runs
+ * on until the process ends.  The call itself allocates and frees nothing.
+ *  - Inputs whose workspace (mgpu_hip_segreduce_workspace_bytes) exceeds that
+ *    size are rejected with hipErrorOutOfMemory (2) and nothing is enqueued;
+ *    count + num_segments up to 2^28 always fits.
+ *  - The device `stream` belongs to must be the current device.
+ *  - All calls on one GPU share the one array: two calls may not overlap in
+ *    time on the same GPU (different streams, or graphs replayed
+ *    concurrently), they would race on it.  Calls on one stream are ordered
+ *    and need nothing else. */
+#define MGPU_HIP_STATIC_SCRATCH_BYTES (4u << 20)
+MGPU_HIP_API int mgpu_hip_segreduce_static(const void* input, int count,
+  const int* segments, int num_segments, void* output, int dtype, int op,
+  const void* init, mgpu_stream_t stream);
+
 /* Same, running only the selected phases (MGPU_PHASE_*).  A later phase uses
  * what an earlier complete call left in the same workspace.  For timing the
  * partition, tile and spine kernels separately. */

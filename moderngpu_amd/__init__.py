@@ -13,5 +13,6 @@ from .ops import (  # noqa: F401
     binary_search_partitions, segreduce_tile_size, lbs_tile_size, lbs_search_tile_size, MgpuError,
     scan, reduce, lbs_segreduce_seg_plus_rank, workcreate,
     sorted_search, inner_join, prepare_segreduce, prepare_load_balance_search,
+    segreduce_static,
 )
 from ._native import lib, library_path  # noqa: F401

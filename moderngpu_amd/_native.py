@@ -21,6 +21,7 @@ SIGNATURES = {
     "mgpu_hip_binary_search_partitions": (c_int, [c_vp, c_int, c_int, c_int, c_int, c_vp, c_vp]),
     "mgpu_hip_segreduce_workspace_bytes": (c_size, [c_int, c_int, c_int]),
     "mgpu_hip_segreduce": (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_int, c_vp, c_vp, c_size, c_vp]),
+    "mgpu_hip_segreduce_static": (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_int, c_vp, c_vp]),
     "mgpu_hip_segreduce_phases": (c_int, [c_vp, c_int, c_vp, c_int, c_vp, c_int, c_int, c_vp, c_vp, c_size, c_vp, c_int]),
     "mgpu_hip_transform_segreduce_mod13": (c_int, [c_int, c_vp, c_int, c_vp, c_int, c_vp, c_size, c_vp]),
     "mgpu_hip_lbs_segreduce_seg_plus_rank": (c_int, [c_int, c_vp, c_int, c_vp, c_int, c_vp, c_size, c_vp]),

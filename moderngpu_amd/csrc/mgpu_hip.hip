@@ -2,11 +2,40 @@
 // and spmv.  Declarations and the reference citations are in
 // include/mgpu_hip.h.
 #include "launcher_common.hxx"
+#include <atomic>
 
 using namespace mgpu;
 using namespace mgpu_hip;
 
+// Device memory of mgpu_hip_segreduce_static: what mgpu_hip_segreduce takes
+// as its workspace argument (tile splits and one carry per tile), held by the
+// library itself so that the call allocates nothing.  Every GPU the library
+// runs on has its own copy at its own address; host code may only use the
+// address hipGetSymbolAddress returns, never the symbol's name.
+static __device__ __align__(256) unsigned char scratch[MGPU_HIP_STATIC_SCRATCH_BYTES];
+
 namespace {
+
+// Address of `scratch` on the current device, looked up once per device.
+enum { max_scratch_devices = 64 };
+std::atomic<void*> scratch_address[max_scratch_devices];
+
+int static_scratch(void** address) {
+  int device = -1;
+  hipError_t result = hipGetDevice(&device);
+  if(hipSuccess != result) return (int)result;
+  if(device < 0 || device >= max_scratch_devices)
+    return (int)hipErrorInvalidDevice;
+  void* p = scratch_address[device].load(std::memory_order_acquire);
+  if(!p) {
+    result = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+    if(hipSuccess != result) return (int)result;
+    if(!p) return (int)hipErrorInvalidSymbol;
+    scratch_address[device].store(p, std::memory_order_release);
+  }
+  *address = p;
+  return (int)hipSuccess;
+}
 
 template<typename type_t>
 int segreduce_any(const void* input, int count, const int* segments,
@@ -171,6 +200,24 @@ int mgpu_hip_segreduce(const void* input, int count, const int* segments,
   void* workspace, size_t workspace_bytes, mgpu_stream_t stream) {
   return mgpu_hip_segreduce_phases(input, count, segments, num_segments,
     output, dtype, op, init, workspace, workspace_bytes, stream,
+    MGPU_PHASE_ALL);
+}
+
+int mgpu_hip_segreduce_static(const void* input, int count,
+  const int* segments, int num_segments, void* output, int dtype, int op,
+  const void* init, mgpu_stream_t stream) {
+  if(!sizes_ok(count, num_segments) || !value_size(dtype))
+    return (int)hipErrorInvalidValue;
+  size_t need = mgpu_hip_segreduce_workspace_bytes(count, num_segments, dtype);
+  if(need > (size_t)MGPU_HIP_STATIC_SCRATCH_BYTES)
+    return (int)hipErrorOutOfMemory;
+  void* workspace = nullptr;
+  int result = static_scratch(&workspace);
+  if(result) return result;
+  // Every piece of the workspace is written by the call before it is read,
+  // so what an earlier call left there needs no clearing.
+  return mgpu_hip_segreduce_phases(input, count, segments, num_segments,
+    output, dtype, op, init, workspace, MGPU_HIP_STATIC_SCRATCH_BYTES, stream,
     MGPU_PHASE_ALL);
 }
 

@@ -107,6 +107,25 @@ def segreduce(values, segments, op="plus", init=0, out=None, unsigned=False,
     return out
 
 
+def segreduce_static(values, segments, op="plus", init=0, out=None, unsigned=False):
+    """segreduce() through the entry point that allocates nothing: its
+    temporaries live in a device array inside the library (4 MiB per GPU).
+    Larger inputs raise MgpuError(2).  Calls on one GPU must not overlap."""
+    _dev_i32(segments, "segments")
+    if not values.is_cuda or not values.is_contiguous():
+        raise TypeError("values must be a contiguous CUDA tensor")
+    code = _dtype_code(values, unsigned)
+    count, nseg = values.numel(), segments.numel()
+    if out is None:
+        out = torch.empty(nseg, dtype=values.dtype, device=values.device)
+    init_c = _CTYPE[code](init)
+    with torch.cuda.device(values.device):
+        _check(lib().mgpu_hip_segreduce_static(
+            _ptr(values), count, _ptr(segments), nseg, _ptr(out), code, OPS[op],
+            ctypes.byref(init_c), _stream()))
+    return out
+
+
 def prepare_segreduce(values, segments, op="plus", init=0, out=None, unsigned=False,
                       phases=7):
     """segreduce() for a caller that repeats one call: arguments are checked
