@@ -84,7 +84,10 @@ struct chunk_width_t {
 // store kernel, but measured slower for these kernels, which read and write
 // at the same time.)  The grid must be xcd_grid(num_tiles); CTAs whose tile
 // is >= num_tiles have nothing to do.
-enum { num_xcds = 8, xcd_run = 16 };
+#ifndef MGPU_XCD_RUN
+#define MGPU_XCD_RUN 16
+#endif
+enum { num_xcds = 8, xcd_run = MGPU_XCD_RUN };
 MGPU_HOST_DEVICE int xcd_grid(int num_tiles) {
   return div_up(num_tiles, (int)(num_xcds * xcd_run)) * (num_xcds * xcd_run);
 }
@@ -127,6 +130,13 @@ MGPU_DEVICE inline merge_range_t tile_range(int count, int num_segments,
 // merged elements, so tiles cut at multiples of lbs_tile_spacing(nv) =
 // nv - lbs_snap_slack never exceed nv elements.
 enum { lbs_snap_items = 32, lbs_snap_window = 32, lbs_snap_slack = 64 };
+
+// Segment starts per block of the coarse partition (lbs_block_partition_f in
+// search.hxx, cta_load_balance_t::fill_blocks below).
+#ifndef MGPU_LBS_BLOCK
+#define MGPU_LBS_BLOCK 256
+#endif
+enum { lbs_block = MGPU_LBS_BLOCK };
 
 MGPU_HOST_DEVICE constexpr int lbs_tile_spacing(int nv) {
   return nv >= 8 * lbs_snap_slack ? nv - lbs_snap_slack : nv;
@@ -452,8 +462,22 @@ struct cta_load_balance_t {
     }
     __syncthreads();
 
-    // 4. running maximum along the items: vt slots per thread in registers,
-    // one exclusive max-scan over the thread totals.
+    // 4. running maximum along the items.
+    scan_slots(tid, a_count, slots, storage.scan);
+  }
+
+  // Running maximum along the item slots: vt slots per thread in registers,
+  // one exclusive max-scan over the thread totals.  Ends with a barrier.
+  MGPU_DEVICE static void scan_slots(int tid, int a_count, int* slots,
+    typename scan_t::storage_t& scan_storage) {
+    scan_slots(tid, a_count, slots, scan_storage, []MGPU_DEVICE() { });
+  }
+  // before_barrier() is called ahead of the final barrier: LDS writes the
+  // caller wants covered by it.
+  template<typename before_barrier_t>
+  MGPU_DEVICE static void scan_slots(int tid, int a_count, int* slots,
+    typename scan_t::storage_t& scan_storage,
+    before_barrier_t before_barrier) {
     int x[vt];
     PRAGMA_UNROLL
     for(int c = 0; c < chunks; ++c) {
@@ -466,7 +490,7 @@ struct cta_load_balance_t {
     PRAGMA_UNROLL
     for(int i = 1; i < vt; ++i) x[i] = max(x[i - 1], x[i]);
 
-    scan_result_t<int> carry = scan_t().scan(tid, x[vt - 1], storage.scan,
+    scan_result_t<int> carry = scan_t().scan(tid, x[vt - 1], scan_storage,
       nt, maximum_t<int>(), 0, scan_type_exc);
 
     PRAGMA_UNROLL
@@ -479,7 +503,222 @@ struct cta_load_balance_t {
         detail::lds_store_chunk<W>(
           slots + layout_t::index(vt * tid + W * c), chunk);
     }
+    before_barrier();
     __syncthreads();
+  }
+
+  //////////////////////////////////////////////////////////////////////////////
+  // Decoding a tile from coarse splits (detail::lbs_block_partition_f): the
+  // partition kernel only says in which block of lbs_block starts each of the
+  // tile's two splits lies.  The tile loads the starts of those blocks and of
+  // everything between them -- its own starts plus at most a block at either
+  // end, as aligned 16-byte loads -- and counts the exact splits itself:
+  // the split of cross-diagonal d has as many starts in front of it as there
+  // are j with segments[j] + j < d.  It then moves both splits back onto a
+  // multiple of lbs_snap_items items where fewer than lbs_snap_window starts
+  // have to move along (see lbs_tile_spacing), which the last lbs_snap_window
+  // starts in front of each split decide; they are among the loaded ones.
+
+  enum {
+    block = detail::lbs_block,
+    lookback = detail::lbs_snap_window,
+    // Starts a tile may load beyond its own: a block at either end, the
+    // look-back, what snapping hands to the tile in front, rounding.
+    block_margin = 2 * block + 2 * lookback - 2,
+    block_extra = block_margin + 10,
+    block_ints = layout_t::capacity(nv) + block_extra,
+    // Rows of nt 16-byte loads held in registers ahead of time.
+    block_rows = (1024 + 4 * nt - 1) / (4 * nt),
+    num_waves = nt / warp_size
+  };
+
+  struct block_storage_t {
+    // Item slots from the bottom (padded layout), the loaded starts at the
+    // top: start j at indices[block_ints - round_up(je - jb, 4) + j - jb].
+    alignas(16) int indices[block_ints];
+    alignas(16) int below[2 * num_waves];   // per wavefront: starts in front
+                                            // of the tile's two diagonals
+    typename scan_t::storage_t scan;
+  };
+
+  struct block_tile_t {
+    int tile;
+    int d0, d1;             // cross-diagonals at the tile's two ends
+    int jb, je;             // starts [jb, je) are loaded
+    bool ahead;             // ... into these registers, ahead of time
+    int starts[block_rows][4];
+  };
+
+  // Loads starts j .. j + 3 (those below end).
+  template<typename segments_it>
+  MGPU_DEVICE static void load_starts(segments_it segments, int j, int end,
+    int (&x)[4]) {
+    if constexpr(std::is_same<segments_it, const int*>::value ||
+      std::is_same<segments_it, int*>::value) {
+      if(j + 4 <= end) {
+        typedef int v4_t __attribute__((ext_vector_type(4), aligned(4)));
+        v4_t v = *(const v4_t*)(segments + j);
+        x[0] = v[0]; x[1] = v[1]; x[2] = v[2]; x[3] = v[3];
+        return;
+      }
+    }
+    PRAGMA_UNROLL
+    for(int e = 0; e < 4; ++e)
+      if(j + e < end) x[e] = (int)segments[j + e];
+  }
+
+  // What a tile has to load, with the loads issued when they fit the
+  // registers set aside for them.
+  template<typename segments_it>
+  MGPU_DEVICE static block_tile_t block_prefetch(int count, int num_segments,
+    int tile, int spacing, const int* blocks, segments_it segments,
+    int tid) {
+    block_tile_t info;
+    int total = count + num_segments;
+    int last_block = max((num_segments + block - 1) / block - 1, 0);
+    info.tile = tile;
+    info.d0 = spacing * tile;
+    info.d1 = info.d0 + min(spacing, total - info.d0);
+    // The clamps only matter for malformed (unsorted) input, which may leave
+    // entries of blocks[] unwritten.
+    int k0 = min(max(blocks[tile], 0), last_block);
+    int k1 = min(max(blocks[tile + 1], k0), last_block);
+    info.jb = max(block * k0 - lookback, 0);
+    info.je = min(min(block * (k1 + 1), num_segments),
+      info.jb + spacing + block_margin + 2);
+    info.ahead = info.je - info.jb <= 4 * nt * block_rows;
+    if(info.ahead) {
+      PRAGMA_UNROLL
+      for(int r = 0; r < block_rows; ++r) {
+        int j = info.jb + 4 * (nt * r + tid);
+        if(j < info.je) load_starts(segments, j, info.je, info.starts[r]);
+      }
+    }
+    return info;
+  }
+
+  // Decodes the tile: leaves, for every item slot p in [0, a_count),
+  // (segment of item - (b_begin - 1)) in storage.indices[index(p)] and returns
+  // the tile's range; starts[rel] is then the start of segment b_begin - 1 +
+  // rel.  snap: whether splits are moved onto multiples of lbs_snap_items
+  // (the tiles must then be cut every nv - lbs_snap_slack).  Ends with a
+  // barrier.
+  template<typename segments_it>
+  MGPU_DEVICE static merge_range_t fill_blocks(const block_tile_t& info,
+    int count, int num_segments, segments_it segments, bool snap, int tid,
+    block_storage_t& storage, const int*& starts) {
+    return fill_blocks(info, count, num_segments, segments, snap, tid,
+      storage, starts, []MGPU_DEVICE() { });
+  }
+  // before_barrier(): see scan_slots().
+  template<typename segments_it, typename before_barrier_t>
+  MGPU_DEVICE static merge_range_t fill_blocks(const block_tile_t& info,
+    int count, int num_segments, segments_it segments, bool snap, int tid,
+    block_storage_t& storage, const int*& starts,
+    before_barrier_t before_barrier) {
+
+    int jb = info.jb, je = info.je;
+    int loaded = je - jb;
+    int* slots = storage.indices;
+    int* staged = storage.indices + (block_ints - ((loaded + 3) & ~3));
+    // The tile's own starts are all but block_margin of the loaded ones at
+    // least, which bounds its items.
+    int a_max = max(nv - max(0, loaded - block_margin), 0);
+
+    // 1. clear the item slots.
+    int zero[W];
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) zero[e] = 0;
+    PRAGMA_UNROLL
+    for(int i = 0; i < chunks; ++i) {
+      int p = W * (nt * i + tid);
+      if(p < a_max)
+        detail::lds_store_chunk<W>(slots + layout_t::index(p), zero);
+    }
+
+    // 2. stage the starts and count those in front of the two diagonals
+    // (start j sits at merged position segments[j] + j).
+    int below0 = 0, below1 = 0;
+    auto stage = [&](int q, const int (&x)[4]) {
+      int j = jb + 4 * q;
+      detail::lds_store_chunk<4>(staged + 4 * q, x);
+      PRAGMA_UNROLL
+      for(int e = 0; e < 4; ++e) {
+        bool valid = j + e < je;
+        below0 += popc(ballot(valid && x[e] < info.d0 - (j + e)));
+        below1 += popc(ballot(valid && x[e] < info.d1 - (j + e)));
+      }
+    };
+    if(info.ahead) {
+      PRAGMA_UNROLL
+      for(int r = 0; r < block_rows; ++r) {
+        int q = nt * r + tid;
+        if(4 * q < loaded) stage(q, info.starts[r]);
+      }
+    } else {
+      for(int q = tid; 4 * q < loaded; q += nt) {
+        int x[4] = { 0, 0, 0, 0 };
+        load_starts(segments, jb + 4 * q, je, x);
+        stage(q, x);
+      }
+    }
+    if(0 == tid % warp_size) {
+      storage.below[2 * (tid / warp_size)] = below0;
+      storage.below[2 * (tid / warp_size) + 1] = below1;
+    }
+    __syncthreads();
+
+    // 3. the exact splits, then the snapped ones.  Lanes 0-31 look at the
+    // last starts in front of the first split, lanes 32-63 at those in front
+    // of the second; every wavefront does the same.
+    int b0 = jb, b1 = jb;
+    PRAGMA_UNROLL
+    for(int w = 0; w < num_waves; ++w) {
+      b0 += storage.below[2 * w];
+      b1 += storage.below[2 * w + 1];
+    }
+    int a0 = info.d0 - b0, a1 = info.d1 - b1;
+    if(snap) {
+      int lane = tid % warp_size;
+      bool second = lane >= warp_size / 2;
+      int a_snap = second ? a1 - a1 % detail::lbs_snap_items :
+        a0 - a0 % detail::lbs_snap_items;
+      int j = (second ? b1 : b0) - 1 - lane % (warp_size / 2);
+      bool above = j >= jb && j < je && staged[j - jb] > a_snap;
+      lanemask_t mask = ballot(above);
+      int back0 = popc((unsigned)mask);
+      int back1 = popc((unsigned)(mask >> 32));
+      if(info.d0 > 0 && back0 < lookback) {
+        a0 -= a0 % detail::lbs_snap_items;
+        b0 -= back0;
+      }
+      if(info.d1 < count + num_segments && back1 < lookback) {
+        a1 -= a1 % detail::lbs_snap_items;
+        b1 -= back1;
+      }
+    }
+    // For well-formed input these change nothing.
+    a0 = min(max(a0, 0), count);
+    a1 = min(max(a1, a0), min(count, a0 + a_max));
+    b0 = min(max(b0, jb), je);
+    b1 = min(max(b1, b0), je);
+    merge_range_t range { a0, a1, b0, b1 };
+    int a_count = a1 - a0;
+
+    // 4. one marker per segment that owns items here (see fill()).
+    for(int j = b0 + tid; j < b1; j += nt) {
+      int s0 = staged[j - jb];
+      int s1 = (j + 1 < b1) ? staged[j + 1 - jb] : 0x7fffffff;
+      int p = s0 - a0;
+      if(s0 != s1 && p >= 0 && p < a_count)
+        slots[layout_t::index(p)] = j - b0 + 1;
+    }
+    __syncthreads();
+
+    // 5. running maximum along the items.
+    scan_slots(tid, a_count, slots, storage.scan, before_barrier);
+    starts = staged + (b0 - 1 - jb);
+    return range;
   }
 
   // The CTA-level search with everything the reference's returns
@@ -583,6 +822,40 @@ struct cached_segment_load_t {
     return staged ? storage.data[rel] : mgpu::load(iterators, max(seg, 0));
   }
 
+  // For tiles decoded from coarse splits (cta_load_balance_t::fill_blocks):
+  // the values of the segments whose starts the tile loads, held in LDS at
+  // (segment - first loaded segment) when there are at most block_capacity
+  // of them.  fetch4() reads the values of four consecutive segments from j
+  // on (those below end) into registers, stage4() puts them at 4 * q ... in
+  // LDS (the caller places the barrier).
+  enum { block_capacity = sizeof(value_t) <= 8 ? 2 * nt : nt };
+  struct block_storage_t {
+    alignas(16) value_t data[block_capacity];
+  };
+  MGPU_DEVICE static void fetch4(int j, int end, pointers_t iterators,
+    value_t (&x)[4]) {
+    if(j + 4 <= end) {
+      PRAGMA_UNROLL
+      for(int e = 0; e < 4; ++e) x[e] = mgpu::load(iterators, j + e);
+    } else {
+      PRAGMA_UNROLL
+      for(int e = 0; e < 4; ++e)
+        if(j + e < end) x[e] = mgpu::load(iterators, j + e);
+    }
+  }
+  MGPU_DEVICE static void stage4(int q, int count, const value_t (&x)[4],
+    block_storage_t& storage) {
+    if(4 * q < count && 4 * q + 4 <= block_capacity) {
+      PRAGMA_UNROLL
+      for(int e = 0; e < 4; ++e) storage.data[4 * q + e] = x[e];
+    }
+  }
+  MGPU_DEVICE static value_t get_block(bool staged, int at, int seg,
+    const block_storage_t& storage, pointers_t iterators) {
+    return staged ? storage.data[max(at, 0)] :
+      mgpu::load(iterators, max(seg, 0));
+  }
+
   // range = segments the tile's items can belong to.
   template<int vt0, int vt>
   MGPU_DEVICE static array_t<value_t, vt> load(int tid, int count,
@@ -621,6 +894,15 @@ struct cached_segment_load_t<nt, tuple<> > {
   MGPU_DEVICE static void commit(int, int, int, const value_t&, storage_t&) {
   }
   MGPU_DEVICE static value_t get(bool, int, int, const storage_t&, tuple<>) {
+    return value_t();
+  }
+  enum { block_capacity = 0 };
+  typedef empty_t block_storage_t;
+  MGPU_DEVICE static void fetch4(int, int, tuple<>, value_t (&)[4]) { }
+  MGPU_DEVICE static void stage4(int, int, const value_t (&)[4],
+    block_storage_t&) { }
+  MGPU_DEVICE static value_t get_block(bool, int, int,
+    const block_storage_t&, tuple<>) {
     return value_t();
   }
 

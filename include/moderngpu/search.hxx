@@ -7,6 +7,7 @@
 #include "loadstore.hxx"
 #include "operators.hxx"
 #include "cta_search.hxx"
+#include "cta_load_balance.hxx"
 #include "memory.hxx"
 #include "context.hxx"
 #include "launcher.hxx"
@@ -270,6 +271,72 @@ struct lbs_partition_scatter_f {
   }
 };
 
+// Coarse splits for the load-balancing search.  The segment starts are looked
+// at in blocks of lbs_block: only the first start of every block is read
+// (one 4-byte load per lbs_block * 4 bytes of starts, so this kernel moves a
+// few per cent of what one pass over the starts would), and for every tile
+// boundary B the kernel records the block in which the boundary's split falls:
+//   blocks[B] = k  <=>  the number c of starts in front of cross-diagonal
+//   spacing * B lies in [lbs_block * k + 1, lbs_block * (k + 1)],
+// (blocks[0] = 0, where c = 0).  The tile kernel reads the starts of its two
+// blocks anyway -- they are its own starts plus at most a block at either end
+// -- and counts its exact splits from them (cta_load_balance_t::fill_blocks).
+// Same scatter idea as above: merged position of block k's first start is
+// s_k = segments[lbs_block * k] + lbs_block * k, and boundary B belongs to
+// block k iff s_k < spacing * B <= s_{k + 1}.
+template<int nt, typename segments_it>
+struct lbs_block_partition_f {
+  enum { direct = 8 };
+  segments_it segments;
+  int num_segments;
+  int count;
+  int spacing;
+  int_divider_t by_spacing;
+  int* blocks;
+
+  MGPU_DEVICE int sample(int k) const {
+    int total = count + num_segments;
+    int j = lbs_block * k;
+    // The clamp keeps malformed input from writing outside blocks[].
+    return j < num_segments ? min(max((int)segments[j] + j, 0), total) : total;
+  }
+
+  MGPU_DEVICE void operator()(int tid, int cta) const {
+    int total = count + num_segments;
+    int num_blocks = div_up(num_segments, (int)lbs_block);
+    int k = nt * cta + tid;
+    int first = 0, n = 0;
+    if(k < num_blocks) {
+      int t0 = by_spacing.div(sample(k));
+      int t1 = by_spacing.div(sample(k + 1));
+      first = t0 + 1;
+      n = t1 - t0;
+    }
+    // Boundaries first .. first + n - 1 lie in block k: written by the thread
+    // when there are few, by the whole wavefront when a segment of the block
+    // spans many tiles.
+    if(n > 0 && n <= direct)
+      for(int i = 0; i < n; ++i) blocks[first + i] = k;
+    int lane = tid % warp_size;
+    lanemask_t spanning = ballot(n > direct);
+    while(spanning) {
+      int src = (int)__builtin_ctzll(spanning);
+      spanning &= spanning - 1;
+      int src_first = readlane(first, src);
+      int src_n = readlane(n, src);
+      int src_k = readlane(k, src);
+      for(int i = lane; i < src_n; i += warp_size)
+        blocks[src_first + i] = src_k;
+    }
+    if(!cta && !tid) {
+      blocks[0] = 0;
+      // The last boundary is the end of the merge whether or not it is a
+      // multiple of the spacing: every start lies in front of it.
+      blocks[div_up(total, spacing)] = max(num_blocks - 1, 0);
+    }
+  }
+};
+
 } // namespace detail
 
 // Writes div_up(a_count + b_count, spacing) + 1 splits into p (device
@@ -336,6 +403,28 @@ int load_balance_partitions_snapped(int count, segments_it segments,
     f { segments, num_segments, count, spacing,
       detail::int_divider_t::make(spacing), p };
   cta_launch<nt>(f, div_up(num_segments, nt * vt), context);
+  return num_partitions;
+}
+
+// The coarse splits of lbs_block_partition_f: div_up(count + num_segments,
+// spacing) + 1 ints.
+template<typename segments_it>
+int load_balance_block_partitions(int count, segments_it segments,
+  int num_segments, int spacing, int* blocks, context_t& context) {
+  enum { nt = 256 };
+  int64_t total = (int64_t)count + num_segments;
+  if(total >= ((int64_t)1 << 31))
+    throw cuda_exception_t(hipErrorInvalidValue);
+  int num_partitions = (int)div_up(total, (int64_t)spacing) + 1;
+  if(!num_segments) {
+    transform<256>([=]MGPU_DEVICE(int index) { blocks[index] = 0; },
+      num_partitions, context);
+    return num_partitions;
+  }
+  detail::lbs_block_partition_f<nt, segments_it> f { segments, num_segments,
+    count, spacing, detail::int_divider_t::make(spacing), blocks };
+  cta_launch<nt>(f, div_up(div_up(num_segments, (int)detail::lbs_block),
+    (int)nt), context);
   return num_partitions;
 }
 

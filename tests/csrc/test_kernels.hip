@@ -275,6 +275,17 @@ API int tk_shfl(const int* in, int* out, int mode, int offset, int width) {
   return finish();
 }
 
+// The coarse partition of the load-balancing search: the block of starts in
+// which each tile boundary's split falls.
+API int tk_lbs_block_partitions(int count, const int* segments,
+  int num_segments, int spacing, int* blocks) {
+  bare_context_t context;
+  load_balance_block_partitions(count, segments, num_segments, spacing,
+    blocks, context);
+  return finish();
+}
+API int tk_lbs_block(void) { return (int)detail::lbs_block; }
+
 API int tk_load_balance(int nt, int vt, int count, const int* segments,
   int num_segments, int* partitions, int* a_index, int* b_index,
   int* merge_flags, int* indices, int* segs, int* ranks, int* ranges,

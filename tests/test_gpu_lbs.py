@@ -33,6 +33,38 @@ def test_partitions_golden_and_oracle(dev, oracle):
         assert np.array_equal(got, oracle.lbs_partitions(count, segs, spacing))
 
 
+def test_block_partitions(dev, oracle):
+    """The coarse partition the search kernels use: for every tile boundary the
+    block of lbs_block starts that holds its split, i.e. (starts in front of
+    the boundary - 1) // lbs_block, against the oracle's exact splits."""
+    import ctypes
+    import torch
+    tk = ctypes.CDLL(os.path.join(os.path.dirname(__file__), "csrc", "libmgpu_test_kernels.so"))
+    block = tk.tk_lbs_block()
+    rng = np.random.default_rng(21)
+    cases = []
+    for _ in range(10):
+        count = int(rng.integers(0, 400000))
+        cases.append((count, random_segments(rng, count, int(rng.integers(1, 60000))),
+                      int(rng.choice([64, 448, 4032, 8128]))))
+    # one segment spanning very many tiles; many empty segments; one start
+    cases.append((3_000_000, np.array([0, 5, 2_999_990], np.int32), 448))
+    cases.append((100, np.zeros(5000, np.int32), 64))
+    cases.append((77, np.array([0], np.int32), 64))
+    for count, segs, spacing in cases:
+        total = count + segs.size
+        n = (total + spacing - 1) // spacing + 1
+        got = torch.full((n,), -7, dtype=torch.int32, device="cuda")
+        d_segs = _dev(segs)
+        assert tk.tk_lbs_block_partitions(count, ctypes.c_void_p(d_segs.data_ptr()), segs.size,
+                                          spacing, ctypes.c_void_p(got.data_ptr())) == 0
+        mp = oracle.lbs_partitions(count, segs, spacing).astype(np.int64)
+        diag = np.minimum(np.arange(n, dtype=np.int64) * spacing, total)
+        in_front = diag - mp                      # starts in front of each boundary
+        want = np.maximum(in_front - 1, 0) // block
+        assert np.array_equal(got.cpu().numpy(), want), (count, segs.size, spacing)
+
+
 def test_merge_path_and_binary_search_partitions(dev, oracle):
     import moderngpu_amd as m
     rng = np.random.default_rng(12)
