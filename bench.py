@@ -30,6 +30,20 @@ def _dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
+_last_config = {}
+
+
+def _config(name, **kwargs):
+    """workloads.<name>(**kwargs), keeping the most recent result: workloads
+    measured one after the other on the same configuration generate it once."""
+    from moderngpu_amd import workloads
+    key = (name, tuple(sorted(kwargs.items())))
+    if key not in _last_config:
+        _last_config.clear()
+        _last_config[key] = getattr(workloads, name)(**kwargs)
+    return _last_config[key]
+
+
 class Workload:
     """name, algorithmic bytes/items per step, device copies, step(i),
     tiles(i) (dominant kernel only), parity check and CPU baseline."""
@@ -93,8 +107,7 @@ def make_c2(copies):
 def make_c3(copies, expand=False):
     import torch
     import moderngpu_amd as m
-    from moderngpu_amd import workloads
-    w = workloads.config3()
+    w = _config("config3")
     n, s = w["count"], w["segments"].size
     segs = [_dev(w["segments"]) for _ in range(copies)]
     vals = [_dev(w["values"]) for _ in range(copies)]
@@ -273,8 +286,7 @@ def make_search(copies, kind):
 def make_c4(copies):
     import torch
     import moderngpu_amd as m
-    from moderngpu_amd import workloads
-    w = workloads.config4()
+    w = _config("config4")
     nnz, rows = w["nnz"], w["segments"].size
     mats = [_dev(w["matrix"]) for _ in range(copies)]
     cols = [_dev(w["columns"]) for _ in range(copies)]
@@ -306,6 +318,30 @@ def make_c4(copies):
         from oracle import oracle
         return lambda: oracle.spmv(w["matrix"], w["columns"], w["vector"], w["segments"])
     wk.cpu = cpu
+    return wk
+
+
+def make_c4_gather_probe(copies):
+    """Not a kernel of this library: torch's index_select over the column
+    indices of configs[3], y[i] = x[columns[i]] -- the same 2^26 gathers into
+    the same 16 MiB vector as spmv does, and nothing else but one store per
+    gather.  A yardstick for the device's gather rate."""
+    import torch
+    w = _config("config4")
+    nnz, rows = w["nnz"], w["segments"].size
+    cols = [_dev(w["columns"]) for _ in range(copies)]
+    x = _dev(w["vector"])
+    outs = [torch.empty(nnz, dtype=torch.float32, device="cuda") for _ in range(copies)]
+    wk = Workload()
+    wk.key, wk.dtype, wk.items = "c4_gather_probe_f32", "f32", nnz
+    wk.name = "torch.index_select(x, columns): %d gathers into 2^22 floats" % nnz
+    wk.bytes = nnz * 4 + nnz * 4 + rows * 4
+    wk.kernel = "torch index_select (yardstick, not part of the library)"
+    wk.step = lambda i: torch.index_select(x, 0, cols[i % copies], out=outs[i % copies])
+    wk.tiles = wk.step
+    wk.check = lambda: bool(np.array_equal(wk.step(0).cpu().numpy(),
+                                           w["vector"][w["columns"]]))
+    wk.cpu = lambda: (lambda: w["vector"][w["columns"]])
     return wk
 
 
@@ -485,20 +521,29 @@ FACTORIES = {
     "sorted_search_i32": lambda c: make_search(c, "search"),
     "inner_join_i32": lambda c: make_search(c, "join"),
     "c4_spmv_f32": make_c4,
+    "c4_gather_probe_f32": make_c4_gather_probe,
     "c5_f64max": lambda c: make_c5(c, "f64max"),
     "c5_i64sum": lambda c: make_c5(c, "i64sum"),
 }
 
-# HBM traffic of the dominant kernel per launch, from rocprofv3 --pmc
-# FETCH_SIZE / WRITE_SIZE runs (profiles/), scaled by what the same counters
-# read for a plain copy of known size.  None until measured.
-TRAFFIC_BYTES = {
-    # profiles/segreduce_tile_f__c2_segreduce_f32.md: FETCH 134,994.4 KiB x 2.000
-    # + WRITE 4,255.6 KiB x 1.000
-    "c2_segreduce_f32": int((134994.4 * 2.000 + 4255.6) * 1024),
-    # profiles/transform_lbs_f__c3_load_balance_search.md
-    "c3_load_balance_search": int((33878.7 * 2.000 + 1048576.0) * 1024),
-}
+def traffic_table():
+    """HBM bytes per launch of each workload's dominant kernel, from the table
+    in profiles/hbm_traffic.md: rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (KiB per
+    dispatch), each scaled by what the same counter reads for a plain copy of
+    known size.  A workload without a row reports null."""
+    table = {}
+    path = os.path.join(ROOT, "profiles", "hbm_traffic.md")
+    if not os.path.exists(path):
+        return table
+    for line in open(path):
+        cells = [c.strip() for c in line.strip().strip("|").split("|")]
+        if len(cells) >= 6 and cells[0] in FACTORIES:
+            try:
+                fetch, ff, write, wf = (float(c.replace(",", "")) for c in cells[2:6])
+            except ValueError:
+                continue
+            table[cells[0]] = int((fetch * ff + write * wf) * 1024)
+    return table
 
 
 def time_steps(fn, steps, warmup):
@@ -511,6 +556,25 @@ def time_steps(fn, steps, warmup):
         fn(warmup + i)
     torch.cuda.synchronize()
     return (time.perf_counter() - t0) / steps
+
+
+def time_each_step(fn, steps, warmup):
+    """Device time of every single step: one HIP event pair per step on the
+    stream the kernels run on.  Returns the sorted list in seconds."""
+    import torch
+    for i in range(warmup):
+        fn(i)
+    torch.cuda.synchronize()
+    pairs = []
+    for i in range(steps):
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        fn(warmup + i)
+        e1.record()
+        pairs.append((e0, e1))
+    torch.cuda.synchronize()
+    return sorted(a.elapsed_time(b) / 1e3 for a, b in pairs)
 
 
 def time_kernel_events(fn, steps, warmup):
@@ -542,10 +606,11 @@ def _time_cpu(run, budget_s):
     return t_total / reps, reps
 
 
-def cpu_baseline(wk, budget_s=4.0):
+def cpu_baseline(wk, budget_s, all_cores):
     """The CPU checker's loop timed on this host: single thread (what the
-    reference's own tests run) and, where the workload splits by segment
-    ranges, all the cores this process may use."""
+    reference's own tests run) and, for the headline workload, all the cores
+    this process may use (contiguous segment ranges per thread).  Every
+    repetition covers the whole workload; repetitions stop after budget_s."""
     sec1, reps1 = _time_cpu(wk.cpu(), budget_s)
     res = {"value": wk.bytes / sec1 / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
            "items_per_s": wk.items / sec1,
@@ -554,7 +619,7 @@ def cpu_baseline(wk, budget_s=4.0):
     make = getattr(wk, "cpu_threads", None)
     cores = len(os.sched_getaffinity(0)) if hasattr(os, "sched_getaffinity") else 1
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores) or cores))
-    if make is not None and cores > 1:
+    if all_cores and make is not None and cores > 1:
         secn, repsn = _time_cpu(make(cores), budget_s)
         res = {"value": wk.bytes / secn / 1e9, "unit": "GB/s", "cores": cores, "kind": "port",
                "items_per_s": wk.items / secn,
@@ -565,6 +630,12 @@ def cpu_baseline(wk, budget_s=4.0):
     return res
 
 
+# BASELINE.json's configs beside the headline one (configs[1]): configs[0],
+# both halves of configs[2], configs[3], both halves of configs[4].
+DEFAULT_EXTRA = ("c1_segreduce_i32,c3_load_balance_search,c3_interval_expand_i32,"
+                 "c4_spmv_f32,c5_f64max,c5_i64sum")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -573,7 +644,7 @@ def main():
     ap.add_argument("--workload", default="c2_segreduce_f32", choices=sorted(FACTORIES))
     ap.add_argument("--copies", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
-    ap.add_argument("--extra", default="c3_load_balance_search",
+    ap.add_argument("--extra", default=DEFAULT_EXTRA,
                     help="comma-separated further workloads reported under 'others'")
     ap.add_argument("--copy-calibration", action="store_true",
                     help="only run a plain 256 MiB device copy a few times: the kernel of "
@@ -601,58 +672,82 @@ def main():
                           "bytes_written": n * 4, "launches": args.steps}))
         return
 
-    def measure(key, with_cpu):
+    import moderngpu_amd as m
+    import ctypes
+    clock_khz, bus_bits = ctypes.c_int(0), ctypes.c_int(0)
+    m.lib().mgpu_hip_memory_properties(0, ctypes.addressof(clock_khz),
+                                       ctypes.addressof(bus_bits))
+    traffic = traffic_table()
+
+    def measure(key, headline):
         wk = FACTORIES[key](args.copies)
         if not wk.check():
             sys.exit("parity check failed for %s: no throughput reported" % key)
+        # The contract's figure: exactly `steps` steps between two
+        # synchronisations, wall clock.  Beside it the median of the same
+        # number of steps timed one by one with HIP events.
         sec = time_steps(wk.step, args.steps, args.warmup)
+        each = time_each_step(wk.step, max(args.steps, 20), args.warmup)
+        median = each[len(each) // 2]
         ksec = time_kernel_events(wk.tiles, args.steps, args.warmup)
         res = {
             "workload": key, "description": wk.name, "dtype": wk.dtype,
-            "ms_per_step": sec * 1e3, "GBps": wk.bytes / sec / 1e9,
+            "ms_per_step": sec * 1e3, "median_ms_per_step": median * 1e3,
+            "GBps": wk.bytes / sec / 1e9,
             "items_per_s": wk.items / sec,
             "pct_hbm_peak": 100.0 * wk.bytes / sec / 1e9 / HBM_PEAK_GBPS,
+            "pct_hbm_peak_median": 100.0 * wk.bytes / median / 1e9 / HBM_PEAK_GBPS,
             "algorithmic_bytes": wk.bytes,
             "roofline": {
                 "bound": "hbm", "kernel": wk.kernel,
                 "achieved": wk.bytes / ksec / 1e9, "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                 "frac": wk.bytes / ksec / 1e9 / HBM_PEAK_GBPS,
                 "kernel_ms": ksec * 1e3,
-                "traffic": TRAFFIC_BYTES.get(key),
+                "traffic": traffic.get(key),
             },
         }
-        if with_cpu:
-            res["cpu_baseline"] = cpu_baseline(wk)
+        if not args.no_cpu:
+            res["cpu_baseline"] = cpu_baseline(wk, 4.0 if headline else 1.5, headline)
         del wk
         torch.cuda.empty_cache()
         return res
 
     props = torch.cuda.get_device_properties(0)
     device = {"name": props.name, "compute_units": props.multi_processor_count,
-              "hbm_peak_used_GBps": HBM_PEAK_GBPS}
-    # memory clock x bus width, double data rate, as the runtime reports them
-    clock_khz = getattr(props, "memory_clock_rate", 0)
-    bus_bits = getattr(props, "memory_bus_width", 0)
-    if clock_khz and bus_bits:
-        device["hbm_peak_from_device_properties_GBps"] = 2.0 * clock_khz * 1e3 * bus_bits / 8 / 1e9
+              "hbm_peak_used_GBps": HBM_PEAK_GBPS,
+              # hipDeviceProp_t's memory clock and bus width, and clock x 2 x
+              # width / 8, the product mgpu's device_prop_string prints.  The
+              # runtime reports 2,000 MHz x 8,192 bits on MI355X, which that
+              # double-data-rate formula turns into 4,096 GB/s; HBM3E moves
+              # 8 Gb/s per pin (four bits per reported clock), so the fractions
+              # here are taken of the published 8 TB/s.
+              "memory_clock_khz": clock_khz.value, "memory_bus_width_bits": bus_bits.value,
+              "hbm_peak_from_device_properties_GBps":
+                  2.0 * clock_khz.value * 1e3 * bus_bits.value / 8 / 1e9}
 
-    main_res = measure(args.workload, not args.no_cpu)
+    main_res = measure(args.workload, True)
     others = {}
     for key in [k for k in args.extra.split(",") if k and k != args.workload]:
         r = measure(key, False)
-        others[key] = {k: r[k] for k in ("ms_per_step", "GBps", "items_per_s", "pct_hbm_peak")}
-        others[key]["roofline_frac"] = r["roofline"]["frac"]
+        others[key] = {k: r[k] for k in (
+            "description", "dtype", "ms_per_step", "median_ms_per_step", "GBps", "items_per_s",
+            "pct_hbm_peak", "pct_hbm_peak_median", "algorithmic_bytes", "roofline")}
+        if "cpu_baseline" in r:
+            others[key]["cpu_baseline"] = r["cpu_baseline"]
 
     line = {
         "metric": "segreduce_input_GBps", "value": main_res["GBps"], "unit": "GB/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": main_res["ms_per_step"], "higher_is_better": True,
+        "ms_per_step": main_res["ms_per_step"],
+        "median_ms_per_step": main_res["median_ms_per_step"],
+        "higher_is_better": True,
         "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
         "data": "synthetic (seeded numpy PCG64, seed 42), inputs resident in HBM, "
                 "%d rotating copies" % args.copies,
         "config": {"workload": main_res["workload"], "description": main_res["description"],
                    "algorithmic_bytes": main_res["algorithmic_bytes"]},
         "items_per_s": main_res["items_per_s"], "pct_hbm_peak": main_res["pct_hbm_peak"],
+        "pct_hbm_peak_median": main_res["pct_hbm_peak_median"],
         "roofline": main_res["roofline"],
     }
     if "cpu_baseline" in main_res:

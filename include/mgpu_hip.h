@@ -53,6 +53,11 @@ enum { MGPU_PHASE_PARTITION = 1, MGPU_PHASE_TILES = 2, MGPU_PHASE_SPINE = 4,
 MGPU_HIP_API int mgpu_hip_version(void);
 /* Text for a return code (hipGetErrorString). */
 MGPU_HIP_API const char* mgpu_hip_error_string(int code);
+/* Memory clock (kHz) and bus width (bits) of `device` as hipDeviceProp_t
+ * gives them -- the two numbers mgpu::device_prop_string multiplies into a
+ * bandwidth figure (context.hxx:25-28): clock x 2 x width / 8. */
+MGPU_HIP_API int mgpu_hip_memory_properties(int device, int* clock_khz,
+  int* bus_width_bits);
 /* Merged elements (items + segment starts) between consecutive tile splits:
  * what the library uses as `spacing` for segreduce on `dtype`, for the
  * load-balancing-search kernels that carry per-segment values (interval

@@ -12,6 +12,7 @@ c_int, c_i64, c_size, c_vp = ctypes.c_int, ctypes.c_int64, ctypes.c_size_t, ctyp
 SIGNATURES = {
     "mgpu_hip_version": (c_int, []),
     "mgpu_hip_error_string": (ctypes.c_char_p, [c_int]),
+    "mgpu_hip_memory_properties": (c_int, [c_int, c_vp, c_vp]),
     "mgpu_hip_segreduce_tile_size": (c_int, [c_int]),
     "mgpu_hip_lbs_tile_size": (c_int, []),
     "mgpu_hip_lbs_search_tile_size": (c_int, []),

@@ -80,6 +80,17 @@ const char* mgpu_hip_error_string(int code) {
   return hipGetErrorString((hipError_t)code);
 }
 
+int mgpu_hip_memory_properties(int device, int* clock_khz,
+  int* bus_width_bits) {
+  if(!clock_khz || !bus_width_bits) return (int)hipErrorInvalidValue;
+  hipDeviceProp_t prop;
+  hipError_t result = hipGetDeviceProperties(&prop, device);
+  if(hipSuccess != result) return (int)result;
+  *clock_khz = prop.memoryClockRate;
+  *bus_width_bits = prop.memoryBusWidth;
+  return 0;
+}
+
 int mgpu_hip_segreduce_tile_size(int dtype) {
   switch(value_size(dtype)) {
     case 4: return segreduce_launch_t<float>::type::sm_ptx::nt *

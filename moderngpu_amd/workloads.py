@@ -9,7 +9,33 @@ Segment descriptors follow moderngpu's convention: ``segments[s]`` is the index
 of the first item of segment ``s``; ascending; ``segments[0] == 0``; no
 trailing ``count`` entry; equal consecutive starts are empty segments.
 """
+import functools
+import os
+
 import numpy as np
+
+
+def _disk_cached(fn):
+    """With MGPU_WORKLOAD_CACHE naming a directory, a configuration's arrays are
+    kept there as .npz and loaded instead of being generated again (several
+    profiler runs of one workload in a row)."""
+    @functools.wraps(fn)
+    def wrapper(*args, **kwargs):
+        folder = os.environ.get("MGPU_WORKLOAD_CACHE")
+        if not folder:
+            return fn(*args, **kwargs)
+        tag = "_".join([fn.__name__] + [str(a) for a in args] +
+                       ["%s-%s" % kv for kv in sorted(kwargs.items())])
+        path = os.path.join(folder, tag + ".npz")
+        if os.path.exists(path):
+            with np.load(path, allow_pickle=False) as z:
+                return {k: (z[k].item() if z[k].ndim == 0 else z[k]) for k in z.files}
+        out = fn(*args, **kwargs)
+        os.makedirs(folder, exist_ok=True)
+        np.savez(path + ".tmp.npz", **out)
+        os.replace(path + ".tmp.npz", path)
+        return out
+    return wrapper
 
 
 def _starts(lengths):
@@ -64,6 +90,7 @@ def config2_segments(seed=42, scale=1):
     return count, _starts(lengths)
 
 
+@_disk_cached
 def config2(seed=42, scale=1):
     """C2: fp32 sum, 2^26 values uniform [0,1), 2^20 segments with geometric
     lengths (mean 64), ~5% forced empty, total exactly 2^26."""
@@ -73,6 +100,7 @@ def config2(seed=42, scale=1):
     return {"values": values, "segments": starts, "op": "plus", "init": 0.0}
 
 
+@_disk_cached
 def config3(seed=42, scale=1):
     """C3: load-balancing search / interval_expand.  2^24 segments whose
     lengths are Zipf(1.2) on [1, 2^16], scaled (stochastic rounding, so many
@@ -88,6 +116,7 @@ def config3(seed=42, scale=1):
     return {"count": count, "segments": _starts(lengths), "values": values}
 
 
+@_disk_cached
 def config4(seed=42, scale=1):
     """C4: CSR spmv, 2^22 rows, nnz/row = 1 + scaled Zipf(1.5) on [1,4096]
     (mean ~16, at least 1, at most 4096), columns uniform and sorted inside
@@ -124,6 +153,7 @@ def config5_segments(seed=42, scale=1):
     return count, _starts(lengths)
 
 
+@_disk_cached
 def config5(seed=42, scale=1, kind="f64max"):
     """C5: extreme skew.  2^27 values, 2^18 segments: four hold ~2^25 items
     each, every other one is empty or has one item.  kind = 'f64max' (normal
