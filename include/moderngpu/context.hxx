@@ -94,7 +94,13 @@ protected:
   hipEvent_t _timer[2];
   hipEvent_t _event;
 
-  // Cache of released device blocks, keyed by capacity.
+  // Cache of released device blocks, keyed by capacity.  A block handed out
+  // again may still be in use by kernels queued earlier on this context's
+  // stream, so whoever gets it has to touch it through that stream only:
+  // the library's kernels do, and so do to_mem(), from_mem() and
+  // mem_t::clone().  The raw-pointer copies htod()/dtoh()/dtod() run on the
+  // null stream, which a stream created with hipStreamNonBlocking does not
+  // wait for: call synchronize() first when the context has such a stream.
   std::multimap<size_t, void*> _free_blocks;
   std::unordered_map<void*, size_t> _live_blocks;
   size_t _cached_bytes;
@@ -266,18 +272,22 @@ public:
     _size = 0;
   }
 
-  context_t& context() { return *_context; }
+  context_t& context() const { return *_context; }
   size_t size() const { return _size; }
   type_t* data() const { return _pointer; }
   memory_space_t space() const { return _space; }
 
-  // Deep copy in the same memory space.
+  // Deep copy in the same memory space, made on the context's stream and
+  // waited for: either block may be one that kernels queued earlier on that
+  // stream still use.
   mem_t clone() {
     mem_t cloned(size(), context(), space());
     if(size()) {
-      hipError_t result = hipMemcpy(cloned.data(), data(),
+      hipStream_t stream = context().stream();
+      hipError_t result = hipMemcpyAsync(cloned.data(), data(),
         sizeof(type_t) * size(), memory_space_device == space() ?
-          hipMemcpyDeviceToDevice : hipMemcpyHostToHost);
+          hipMemcpyDeviceToDevice : hipMemcpyHostToHost, stream);
+      if(hipSuccess == result) result = hipStreamSynchronize(stream);
       if(hipSuccess != result) throw cuda_exception_t(result);
     }
     return cloned;

@@ -369,6 +369,15 @@ struct lbs_coarse_splits_t {
     0 == tuple_size<pointers_t>::value };
 };
 
+// count + num_segments as the 32-bit total the kernels index with; throws
+// instead of wrapping when the sum does not fit.
+inline int lbs_total(int count, int num_segments) {
+  int64_t total = (int64_t)count + num_segments;
+  if(count < 0 || num_segments < 0 || total >= ((int64_t)1 << 31))
+    throw cuda_exception_t(hipErrorInvalidValue);
+  return (int)total;
+}
+
 enum { lbs_phase_partition = 1, lbs_phase_tiles = 2, lbs_phase_all = 3 };
 
 // Ints of partition storage for `total` merged elements cut into tiles of nv:
@@ -392,7 +401,7 @@ int lbs_partition_tiles(int count, segments_it segments, int num_segments,
   else
     load_balance_partitions_snapped<1, 1>(count, segments, num_segments,
       spacing, pairs, context);
-  return div_up(count + num_segments, spacing);
+  return div_up(lbs_total(count, num_segments), spacing);
 }
 
 // Partition + tile kernels with the partition array in caller-provided
@@ -403,9 +412,10 @@ void transform_lbs_launch(func_t f, int count, segments_it segments,
   int num_segments, pointers_t caching_iterators, int* mp_data, int phases,
   context_t& context, args_t... args) {
 
-  if(count + num_segments <= 0) return;
+  int total = lbs_total(count, num_segments);
+  if(!total) return;
   int nv = launch_t::nv(context);
-  int num_tiles = div_up(count + num_segments, lbs_tile_spacing(nv));
+  int num_tiles = div_up(total, lbs_tile_spacing(nv));
 
   if constexpr(lbs_coarse_splits_t<pointers_t>::value) {
     if(phases & lbs_phase_partition)
@@ -442,9 +452,10 @@ void transform_lbs(func_t f, int count, segments_it segments,
   typedef typename conditional_typedef_t<launch_arg_t,
     typename detail::lbs_launch_select_t<pointers_t>::type_t>::type_t launch_t;
 
-  if(count + num_segments <= 0) return;
-  mem_t<int> mp(detail::lbs_partition_ints(count + num_segments,
-    launch_t::nv(context)), context);
+  int total = detail::lbs_total(count, num_segments);
+  if(!total) return;
+  mem_t<int> mp(detail::lbs_partition_ints(total, launch_t::nv(context)),
+    context);
   detail::transform_lbs_launch<launch_t>(f, count, segments, num_segments,
     caching_iterators, mp.data(), detail::lbs_phase_all, context, args...);
 }

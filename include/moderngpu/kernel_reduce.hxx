@@ -58,7 +58,7 @@ struct reduce_final_f {
   }
 };
 
-enum { reduce_final_nt = 1024, reduce_final_vt = 8, reduce_small_count = 16384 };
+enum { reduce_final_nt = 1024, reduce_small_count = 16384 };
 
 // Partials needed for `count` items in tiles of nv.
 MGPU_HOST_DEVICE size_t reduce_partials_count(int64_t count, int nv) {
@@ -73,8 +73,8 @@ void reduce_launch(input_it input, int count, output_it reduction, op_t op,
   type_t* partials, context_t& context) {
   if(count <= 0) return;
   if(count <= reduce_small_count) {
-    reduce_final_f<reduce_final_nt, reduce_final_vt, input_it, output_it,
-      type_t, op_t>
+    reduce_final_f<reduce_final_nt, spine_vt_t<type_t>::value, input_it,
+      output_it, type_t, op_t>
       k { input, count, reduction, op };
     cta_launch<reduce_final_nt>(k, 1, context);
     return;
@@ -83,8 +83,8 @@ void reduce_launch(input_it input, int count, output_it reduction, op_t op,
   scan_upsweep_f<launch_t, input_it, type_t, op_t>
     up { input, count, op, partials, num_tiles };
   cta_launch<launch_t>(up, xcd_grid(num_tiles), context);
-  reduce_final_f<reduce_final_nt, reduce_final_vt, const type_t*, output_it,
-    type_t, op_t>
+  reduce_final_f<reduce_final_nt, spine_vt_t<type_t>::value, const type_t*,
+    output_it, type_t, op_t>
     k { partials, num_tiles, reduction, op };
   cta_launch<reduce_final_nt>(k, 1, context);
 }

@@ -246,6 +246,17 @@ struct scan_downsweep_f {
   }
 };
 
+// Values per thread of the one-CTA kernels (the spine, and the last step of
+// reduce): 8 for types of up to 8 bytes, fewer for wider ones so that the
+// 1,024-thread tile stays at 64 KB of LDS.
+template<typename type_t>
+struct spine_vt_t {
+  enum {
+    value = sizeof(type_t) <= 8 ? 8 :
+      (64 / sizeof(type_t) > 1 ? 64 / sizeof(type_t) : 1)
+  };
+};
+
 enum {
   scan_spine_nt = 1024, scan_spine_vt = 8,
   // At most this many items are scanned by the spine CTA alone, and at most
@@ -283,8 +294,8 @@ void scan_launch(input_it input, int count, output_it output, op_t op,
   int nv = launch_t::nv(context);
   if(count <= scan_small_count) {
     // Few items (or none: the reduction is type_t()): one CTA does it all.
-    scan_spine_f<scan_type, scan_spine_nt, scan_spine_vt, input_it,
-      output_it, type_t, op_t, reduction_it>
+    scan_spine_f<scan_type, scan_spine_nt, spine_vt_t<type_t>::value,
+      input_it, output_it, type_t, op_t, reduction_it>
       k { input, count, output, op, reduction };
     cta_launch<scan_spine_nt>(k, 1, context);
     if(event) scan_record(event, context);
@@ -297,8 +308,8 @@ void scan_launch(input_it input, int count, output_it output, op_t op,
   cta_launch<launch_t>(up, xcd_grid(num_tiles), context);
 
   if(num_tiles <= scan_spine_limit) {
-    scan_spine_f<scan_type_exc, scan_spine_nt, scan_spine_vt, const type_t*,
-      type_t*, type_t, op_t, reduction_it>
+    scan_spine_f<scan_type_exc, scan_spine_nt, spine_vt_t<type_t>::value,
+      const type_t*, type_t*, type_t, op_t, reduction_it>
       k { partials, num_tiles, partials, op, reduction };
     cta_launch<scan_spine_nt>(k, 1, context);
   } else {

@@ -24,6 +24,22 @@ inline void throw_on_error(hipError_t status) {
   if(hipSuccess != status) throw cuda_exception_t(status);
 }
 
+// The same copy issued on the context's stream and waited for.  Memory that
+// comes from a context may be a recycled block (standard_context_t keeps
+// released blocks) that kernels queued earlier on the context's stream still
+// use; a copy on the null stream is not ordered behind a non-blocking stream,
+// a copy on the context's stream is.
+template<hipMemcpyKind kind, typename type_t>
+hipError_t copy_elements(type_t* dest, const type_t* source, size_t count,
+  context_t& context) {
+  if(!count) return hipSuccess;
+  hipStream_t stream = context.stream();
+  hipError_t result = hipMemcpyAsync(dest, source, sizeof(type_t) * count,
+    kind, stream);
+  if(hipSuccess != result) return result;
+  return hipStreamSynchronize(stream);
+}
+
 // A mem_t of count elements, element i set to value_at(i) by a kernel.
 template<typename type_t, typename value_at_t>
 mem_t<type_t> mem_from_function(value_at_t value_at, size_t count,
@@ -72,16 +88,19 @@ hipError_t htod(type_t* dest, const std::vector<type_t>& source) {
 // mem_t factories.
 
 // A device copy of a host vector, and back.
+// Both copies run on the context's stream (see detail::copy_elements).
 template<typename type_t>
 mem_t<type_t> to_mem(const std::vector<type_t>& data, context_t& context) {
   mem_t<type_t> mem(data.size(), context);
-  detail::throw_on_error(htod(mem.data(), data));
+  detail::throw_on_error(detail::copy_elements<hipMemcpyHostToDevice>(
+    mem.data(), data.data(), data.size(), context));
   return mem;
 }
 template<typename type_t>
 std::vector<type_t> from_mem(const mem_t<type_t>& mem) {
-  std::vector<type_t> host;
-  detail::throw_on_error(dtoh(host, mem.data(), mem.size()));
+  std::vector<type_t> host(mem.size());
+  detail::throw_on_error(detail::copy_elements<hipMemcpyDeviceToHost>(
+    host.data(), mem.data(), mem.size(), mem.context()));
   return host;
 }
 

@@ -61,14 +61,44 @@ void cta_launch(func_t f, int num_ctas, context_t& context, args_t... args) {
 // The tile count is only known on the device: a fixed grid of several CTAs per
 // resident slot walks the tiles with a grid stride, and a CTA stops at the
 // first tile index at or past *num_tiles.
+namespace detail {
+template<typename func_t>
+struct strided_tiles_f {
+  func_t f;
+  const int* num_tiles;
+  template<typename... args_t>
+  MGPU_DEVICE void operator()(int tid, int cta, args_t... args) {
+    for(int tile = cta, end = *num_tiles; tile < end; tile += (int)gridDim.x)
+      f(tid, tile, args...);
+  }
+};
+} // namespace detail
+
 template<typename launch_box, typename func_t, typename... args_t>
 void cta_launch(func_t f, const int* num_tiles, context_t& context,
   args_t... args) {
-  int grid = 8 * occupancy<launch_box>(f, context);
-  auto strided = [=]MGPU_DEVICE(int tid, int cta, args_t... args) {
-    for(int tile = cta, end = *num_tiles; tile < end; tile += grid)
-      f(tid, tile, args...);
-  };
+  detail::strided_tiles_f<func_t> strided { f, num_tiles };
+  // Resident CTAs of the kernel that is launched (the walking one); a context
+  // that does not fill in its device properties gets the count of compute
+  // units from the runtime.
+  int num_blocks = 0;
+  hipError_t result = hipOccupancyMaxActiveBlocksPerMultiprocessor(
+    &num_blocks,
+    launch_box_cta_k<launch_box, detail::strided_tiles_f<func_t>, args_t...>,
+    detail::box_threads<launch_box>(context), (size_t)0);
+  if(hipSuccess != result) throw cuda_exception_t(result);
+  int num_cus = context.props().multiProcessorCount;
+  if(num_cus <= 0) {
+    int device = 0;
+    result = hipGetDevice(&device);
+    if(hipSuccess == result)
+      result = hipDeviceGetAttribute(&num_cus,
+        hipDeviceAttributeMultiprocessorCount, device);
+    if(hipSuccess != result) throw cuda_exception_t(result);
+  }
+  int grid = 8 * num_cus * num_blocks;
+  // Nothing would run although *num_tiles may be positive.
+  if(grid < 1) throw cuda_exception_t(hipErrorInvalidConfiguration);
   cta_launch<launch_box>(strided, grid, context, args...);
 }
 

@@ -7,6 +7,7 @@
 #include <moderngpu/memory.hxx>
 #include <moderngpu/loadstore.hxx>
 #include <moderngpu/cpp11.hxx>
+#include <moderngpu/kernel_load_balance.hxx>
 #include <cstdio>
 
 using namespace mgpu;
@@ -237,6 +238,81 @@ static int check_bit_helpers(context_t& context) {
   return 0;
 }
 
+// A context on a stream the null stream does not wait for: blocks released
+// while a kernel that writes them is still queued come back from the
+// context's cache at once, and whatever fills them next has to be ordered
+// behind that kernel.
+static int check_nonblocking_stream() {
+  hipStream_t stream;
+  CHECK(hipSuccess == hipStreamCreateWithFlags(&stream, hipStreamNonBlocking));
+  {
+    standard_context_t context(false, stream);
+    int count = 1 << 22;
+    std::vector<int> host(count);
+    for(int round = 0; round < 6; ++round) {
+      int* first = nullptr;
+      {
+        mem_t<int> junk = fill<int>(-1, count, context);
+        first = junk.data();
+      }                                   // released, fill may still run
+      for(int i = 0; i < count; ++i) host[i] = i ^ round;
+      mem_t<int> mem = to_mem(host, context);
+      CHECK(mem.data() == first);         // the recycled block
+      CHECK(from_mem(mem) == host);
+      mem_t<int> copy = mem.clone();
+      CHECK(from_mem(copy) == host);
+    }
+  }
+  CHECK(hipSuccess == hipStreamDestroy(stream));
+  return 0;
+}
+
+// A context that leaves its device properties empty (as one that only wraps a
+// caller's stream may): the launch with a device-side tile count still finds
+// the number of compute units.
+struct bare_props_context_t : standard_context_t {
+  hipDeviceProp_t empty;
+  bare_props_context_t() : standard_context_t(false) {
+    memset(&empty, 0, sizeof(empty));
+  }
+  const hipDeviceProp_t& props() const override { return empty; }
+};
+static int check_launch_without_props() {
+  bare_props_context_t context;
+  int tiles = 3001;
+  mem_t<int> num_tiles = to_mem(std::vector<int> { tiles }, context);
+  mem_t<int> hits = fill<int>(0, 4000, context);
+  int* h = hits.data();
+  cta_launch<launch_params_t<64, 1> >([=]MGPU_DEVICE(int tid, int tile) {
+    if(!tid) atomicAdd(h + tile, 1);
+  }, num_tiles.data(), context);
+  std::vector<int> host = from_mem(hits);
+  for(int i = 0; i < 4000; ++i) CHECK(host[i] == (i < tiles ? 1 : 0));
+  return 0;
+}
+
+// count + num_segments has to fit 31 bits; the call throws instead of
+// wrapping round (nothing is launched, the pointers are never read).
+static int check_index_limit(context_t& context) {
+  bool thrown = false;
+  try {
+    load_balance_search(2147483647, (const int*)nullptr, 10, (int*)nullptr,
+      context);
+  } catch(cuda_exception_t& e) {
+    thrown = hipErrorInvalidValue == e.result;
+  }
+  CHECK(thrown);
+  thrown = false;
+  try {
+    transform_lbs([]MGPU_DEVICE(int, int, int) { }, 2000000000,
+      (const int*)nullptr, 200000000, context);
+  } catch(cuda_exception_t& e) {
+    thrown = hipErrorInvalidValue == e.result;
+  }
+  CHECK(thrown);
+  return 0;
+}
+
 int main() {
   standard_context_t context(false);
   CHECK(0 == check_bit_helpers(context));
@@ -244,6 +320,9 @@ int main() {
   CHECK(0 == check_tile_movement(context));
   CHECK(0 == check_memory(context));
   CHECK(0 == check_tuples(context));
+  CHECK(0 == check_nonblocking_stream());
+  CHECK(0 == check_launch_without_props());
+  CHECK(0 == check_index_limit(context));
   printf("runtime: all passed\n");
   return 0;
 }

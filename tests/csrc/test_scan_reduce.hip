@@ -138,10 +138,47 @@ static int test_reduce_sweep(context_t& context) {
   return 0;
 }
 
+// A 32-byte value type with a non-commutative operator (first tag wins, the
+// four sums add): scan and reduce with the default launch boxes, at a size of
+// one CTA, of a few tiles and of thousands of tiles.
+struct wide_t { int64_t tag; int64_t sum[3]; };
+struct wide_left_t {
+  MGPU_HOST_DEVICE wide_t operator()(wide_t a, wide_t b) const {
+    return wide_t { a.tag, { a.sum[0] + b.sum[0], a.sum[1] + b.sum[1],
+      a.sum[2] + b.sum[2] } };
+  }
+};
+static int test_wide_type(context_t& context) {
+  static_assert(32 == sizeof(wide_t), "");
+  for(int count : { 1, 999, 16384, 16385, 300000, 5000011 }) {
+    std::vector<wide_t> host(count);
+    for(int i = 0; i < count; ++i)
+      host[i] = wide_t { i + 3, { 1, i, -2 } };
+    mem_t<wide_t> in = to_mem(host, context);
+    mem_t<wide_t> out(count, context), red(1, context);
+    scan<scan_type_inc>(in.data(), count, out.data(), wide_left_t(),
+      red.data(), context);
+    std::vector<wide_t> z = from_mem(out);
+    for(int i = 0; i < count; ++i) {
+      int64_t tri = (int64_t)i * (i + 1) / 2;
+      CHECK(z[i].tag == 3 && z[i].sum[0] == i + 1 && z[i].sum[1] == tri &&
+        z[i].sum[2] == -2 * (int64_t)(i + 1), "wide scan, count %d, at %d", count, i);
+    }
+    wide_t r = from_mem(red)[0];
+    CHECK(r.tag == 3 && r.sum[0] == count, "wide scan total, count %d", count);
+    reduce(in.data(), count, red.data(), wide_left_t(), context);
+    r = from_mem(red)[0];
+    CHECK(r.tag == 3 && r.sum[0] == count &&
+      r.sum[1] == (int64_t)count * (count - 1) / 2, "wide reduce, count %d", count);
+  }
+  return 0;
+}
+
 int main() {
   standard_context_t context(false);
   if(test_scan_constant(context) || test_scan_sizes(context) ||
-    test_scan_two_levels(context) || test_reduce_sweep(context))
+    test_scan_two_levels(context) || test_reduce_sweep(context) ||
+    test_wide_type(context))
     return 1;
   printf("scan/reduce: all passed\n");
   return 0;
