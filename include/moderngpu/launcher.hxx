@@ -18,6 +18,8 @@
 //
 // Each helper below returns true when it has made the call.
 #pragma once
+#include <cstdio>
+#include <cstdlib>
 #include "context.hxx"
 #include "memory.hxx"
 #include "operators.hxx"
@@ -85,10 +87,26 @@ inline void launcher_check(int code) {
   if(code) throw cuda_exception_t((hipError_t)code);
 }
 
-// Number of calls that went to the library (for tests).
+// Number of calls that went to the library (for tests).  With the environment
+// variable MGPU_HIP_LAUNCHER_REPORT set, the count is printed to stderr when
+// the program ends ("mgpu launcher calls: N"), and a line when the first call
+// is made (a program that is ended from outside never gets to the other):
+// that is how a program that cannot be edited -- one written for the CUDA
+// library and only recompiled -- shows which way its calls went.
+struct launcher_counter_t {
+  long calls = 0;
+  launcher_counter_t() {
+    if(getenv("MGPU_HIP_LAUNCHER_REPORT"))
+      fprintf(stderr, "mgpu launcher: first call\n");
+  }
+  ~launcher_counter_t() {
+    if(getenv("MGPU_HIP_LAUNCHER_REPORT"))
+      fprintf(stderr, "mgpu launcher calls: %ld\n", calls);
+  }
+};
 inline long& launcher_calls() {
-  static long calls = 0;
-  return calls;
+  static launcher_counter_t counter;
+  return counter.calls;
 }
 
 template<typename launch_arg_t, typename input_it, typename segments_it,

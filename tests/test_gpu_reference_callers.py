@@ -25,13 +25,26 @@ BIN = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))),
                    "oracle", "_ref")
 
 
+# Programs named launcher_* are the same sources built with MGPU_HIP_LAUNCHER:
+# the public templates then call the prebuilt kernels of libmgpu_hip.so where
+# the arguments are ones its C layer covers.  With MGPU_HIP_LAUNCHER_REPORT in
+# the environment such a program says on stderr when its first call goes
+# there and, at exit, how many did.
+_ENV = dict(os.environ, MGPU_HIP_LAUNCHER_REPORT="1")
+
+
 def _run(name, limit=110):
     """Returns (exit status, stdout, stderr)."""
     path = os.path.join(BIN, name)
     if not os.path.exists(path):
         pytest.skip("oracle/_ref/%s was not built (no reference tree at build time)" % name)
-    proc = subprocess.run([path], capture_output=True, text=True, timeout=limit)
+    proc = subprocess.run([path], capture_output=True, text=True, timeout=limit, env=_ENV)
     return proc.returncode, proc.stdout, proc.stderr
+
+
+def _launcher_calls(text):
+    found = re.findall(r"mgpu launcher calls: (\d+)", text)
+    return int(found[-1]) if found else 0
 
 
 def _run_for_a_while(name, seconds, enough=None):
@@ -47,7 +60,8 @@ def _run_for_a_while(name, seconds, enough=None):
     if not os.path.exists(path):
         pytest.skip("oracle/_ref/%s was not built (no reference tree at build time)" % name)
     master, slave = pty.openpty()
-    proc = subprocess.Popen([path], stdout=slave, stderr=slave, stdin=subprocess.DEVNULL)
+    proc = subprocess.Popen([path], stdout=slave, stderr=slave, stdin=subprocess.DEVNULL,
+                            env=_ENV)
     os.close(slave)
     chunks, deadline, code = [], time.time() + seconds, None
     while True:
@@ -90,53 +104,72 @@ def test_reference_test_load_balance(dev, name):
     lines = re.findall(r"^ *(\d+): +(\d+)$", out, flags=re.M)
     assert len(lines) == 200030
     assert lines[-1] == ("200029", str(200029 // 100))
+    if name.startswith("launcher_"):
+        assert _launcher_calls(err) == 1, err[-500:]
 
 
-def test_reference_test_sortedsearch(dev):
+@pytest.mark.parametrize("name", ["test_sortedsearch", "launcher_test_sortedsearch"])
+def test_reference_test_sortedsearch(dev, name):
     # Host asserts on every index (the build does not define NDEBUG).
-    code, out, err = _run("test_sortedsearch")
+    code, out, err = _run(name)
     assert code == 0, err[-2000:]
+    if name.startswith("launcher_"):
+        assert _launcher_calls(err) > 0, err[-500:]
 
 
-def test_reference_test_reduce(dev):
+@pytest.mark.parametrize("name", ["test_reduce", "launcher_test_reduce"])
+def test_reference_test_reduce(dev, name):
     # 1,012 sizes from 1,000 to 23.4 M, reduce<192 x 11> and transform_reduce
-    # against std::accumulate; exit(1) on a mismatch.
-    code, out, err = _run("test_reduce")
+    # against std::accumulate; exit(1) on a mismatch.  Both calls instantiate
+    # in place whatever the build: one names a launch box, the other takes a
+    # lambda.
+    code, out, err = _run(name)
     assert code == 0, out[-2000:] + err[-2000:]
     assert "ERROR" not in out
     assert out.count("success") > 1000
+    assert _launcher_calls(err) == 0
 
 
-def test_reference_test_segreduce(dev):
+@pytest.mark.parametrize("name", ["test_segreduce", "launcher_test_segreduce"])
+def test_reference_test_segreduce(dev, name):
     # 1,000 rounds of 10^8 items, each checked by a host loop: far more than a
     # test run has time for, so it is ended after a while and what it printed
     # until then is checked (it reports a mismatch and calls exit(0)).
     # The gate does not depend on how fast the host is: one complete round
     # without a mismatch passes; the run stops at three rounds or 60 s.
-    code, out = _run_for_a_while("test_segreduce", 60,
+    code, out = _run_for_a_while(name, 60,
                                  enough=lambda text: text.count("passed") >= 3)
     print(out[-400:])
     assert code in (None, 0), out[-2000:]
     assert "error" not in out.lower()
     assert out.count("passed") >= 1, out[-2000:]
+    # Its one call is transform_segreduce over a lambda, which instantiates in
+    # place whatever the build (a call into the library would have announced
+    # itself: the program is ended from outside, so no count is printed).
+    assert "mgpu launcher: first call" not in out
 
 
-def test_reference_test_merge(dev):
+@pytest.mark.parametrize("name", ["test_merge", "launcher_test_merge"])
+def test_reference_test_merge(dev, name):
     # Sizes from 1,000 to 10^8 in steps of 10 %, each merged on the device and
     # with std::merge (the inputs are sorted on the host, which takes most of
     # the time at the large sizes); ended after a while like test_segreduce.
-    # Stops at 80 sizes or 60 s; passes with at least one size and no failure.
-    code, out = _run_for_a_while("test_merge", 60,
-                                 enough=lambda text: text.count("SUCCESS") >= 80)
+    # Stops at 60 sizes or 60 s; passes with at least one size and no failure.
+    # merge is not among the calls the C layer covers: in place either way.
+    code, out = _run_for_a_while(name, 60,
+                                 enough=lambda text: text.count("SUCCESS") >= 60)
     print(out[-400:])
     assert code in (None, 0), out[-2000:]
     assert "FAILURE" not in out
     assert out.count("SUCCESS") >= 1, out[-2000:]
 
 
-def test_reference_test_join_and_intervalexpand(dev):
+@pytest.mark.parametrize("prefix", ["", "launcher_"])
+def test_reference_test_join_and_intervalexpand(dev, prefix):
     for name in ("test_join", "test_intervalexpand"):
-        code, out, err = _run(name)
+        # test_join joins two empty inputs and test_intervalexpand only
+        # creates a context: building and running them is the whole test.
+        code, out, err = _run(prefix + name)
         assert code == 0, name + err[-2000:]
 
 
