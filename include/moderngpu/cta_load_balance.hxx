@@ -77,23 +77,31 @@ struct chunk_width_t {
 // has its own L2.  With tile == blockIdx.x, neighbouring tiles -- which share
 // the cache line where one tile's data ends and the next begins -- always sit
 // on different XCDs: the line is fetched twice, or written back partially by
-// two L2s.  Here each XCD takes runs of xcd_run consecutive tiles, and the
-// runs of the 8 XCDs interleave, so the set of tiles in flight stays one
-// compact window of memory.  (Giving each XCD one contiguous eighth of all
-// tiles merges even more boundary lines and is the fastest layout for a pure
-// store kernel, but measured slower for these kernels, which read and write
-// at the same time.)  The grid must be xcd_grid(num_tiles); CTAs whose tile
-// is >= num_tiles have nothing to do.
-#ifndef MGPU_XCD_RUN
-#define MGPU_XCD_RUN 16
-#endif
-enum { num_xcds = 8, xcd_run = MGPU_XCD_RUN };
+// two L2s.  xcd_tile() gives each XCD runs of xcd_run consecutive tiles, and
+// the runs of the 8 XCDs interleave, so the set of tiles in flight stays one
+// compact window of memory.  xcd_tile_eighths() gives each XCD one contiguous
+// eighth of all tiles.  That is the fastest layout for a kernel that only
+// stores (1 GiB in ragged tiles of about 30 KB: 171 us against 190-200 us
+// with runs or with tile == blockIdx.x), but as soon as each tile also reads
+// a couple of KB that miss the L2 the advantage is gone (all three layouts
+// 195-205 us), and the search kernels measured slower with it (216 against
+// 195 us); the segmented reduce, which reads far more than it writes, takes
+// the same time in its tile kernel and 1.1 us less as a whole call on 2^26
+// floats (49.2 against 50.3 us), so that kernel uses eighths and the others
+// runs.  The grid must be xcd_grid(num_tiles) for either; CTAs whose tile is
+// >= num_tiles have nothing to do.
+enum { num_xcds = 8, xcd_run = 16 };
 MGPU_HOST_DEVICE int xcd_grid(int num_tiles) {
   return div_up(num_tiles, (int)(num_xcds * xcd_run)) * (num_xcds * xcd_run);
 }
 MGPU_DEVICE inline int xcd_tile(int cta, int) {
   int xcd = cta % num_xcds, local = cta / num_xcds;
   return ((local / xcd_run) * num_xcds + xcd) * xcd_run + local % xcd_run;
+}
+MGPU_DEVICE inline int xcd_tile_eighths(int cta, int num_tiles) {
+  int xcd = cta % num_xcds, local = cta / num_xcds;
+  int per = (num_tiles + num_xcds - 1) / num_xcds;
+  return local < per ? xcd * per + local : num_tiles;
 }
 
 // The tile's item and segment ranges from the two splits at its ends, forced

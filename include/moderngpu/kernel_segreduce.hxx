@@ -287,8 +287,8 @@ struct segreduce_tile_f {
 
   template<typename... args_t>
   MGPU_DEVICE void operator()(int tid, int cta, args_t... args) const {
-    // Neighbouring tiles run on the same XCD (see xcd_tile).
-    cta = xcd_tile(cta, num_tiles);
+    // Neighbouring tiles run on the same XCD (see xcd_tile_eighths).
+    cta = xcd_tile_eighths(cta, num_tiles);
     if(cta >= num_tiles) return;
     __shared__ storage_t shared;
 
