@@ -516,6 +516,130 @@ struct cta_load_balance_t {
   }
 
   //////////////////////////////////////////////////////////////////////////////
+  // The same decode in half the LDS: 16-bit slots.  A tile has fewer than
+  // 2^16 elements, so (segment - first segment + 1) fits 16 bits, and so does
+  // the start of every segment that begins inside the tile when it is kept
+  // relative to the tile's first item.  Only the start of the segment that is
+  // open when the tile begins may lie anywhere in front; it is kept apart, as
+  // a 32-bit difference.  With 512 x 12 tiles this is 14 KB instead of 28 KB
+  // per CTA, with 512 x 16 tiles 19 KB instead of 37 KB.
+
+  typedef unsigned short slot_t;
+  static_assert(nv + 2 < 65536, "16-bit tile slots need tiles below 2^16");
+
+  struct compact_storage_t {
+    // Item slots (padded layout), then the relative starts: entry 0 is zero
+    // and stands for the open segment, entry 1 + j belongs to segment
+    // b_begin + j.
+    alignas(16) slot_t slots[layout_t::capacity(nv) + 8];
+    int open_offset;
+    typename scan_t::storage_t scan;
+  };
+
+  // What fill_compact() leaves: slot p holds (segment of tile item p) -
+  // (b_begin - 1), and the rank of item p in that segment is rank(p, rel).
+  struct compact_tile_t {
+    const slot_t* slots;
+    const slot_t* starts;
+    int open_offset;        // first item of the tile - start of open segment
+    MGPU_DEVICE int rank(int p, int rel) const {
+      return p - (int)starts[rel] + (rel ? 0 : open_offset);
+    }
+  };
+
+  template<typename segments_it>
+  MGPU_DEVICE compact_tile_t fill_compact(merge_range_t range,
+    segments_it segments, int tid, compact_storage_t& storage,
+    prefetch_t ahead) const {
+
+    int a_count = range.a_count();
+    int b_count = range.b_count();
+    slot_t* slots = storage.slots;
+    slot_t* starts = storage.slots + starts_offset(a_count);
+
+    // 1. clear the item slots.
+    slot_t zero[W];
+    PRAGMA_UNROLL
+    for(int e = 0; e < W; ++e) zero[e] = 0;
+    PRAGMA_UNROLL
+    for(int i = 0; i < chunks; ++i) {
+      int p = W * (nt * i + tid);
+      if(p < a_count)
+        detail::lds_store_chunk<W>(slots + layout_t::index(p), zero);
+    }
+
+    // 2. stage the segment starts of the tile, relative to its first item
+    // (a start of well-formed input lies in [a_begin, a_end]; the clamp is
+    // for anything else).
+    auto relative = [&](int start) {
+      return (slot_t)min(max(start - range.a_begin, 0), 65535);
+    };
+    int preceding = 0;
+    if(ahead.valid) {
+      PRAGMA_UNROLL
+      for(int r = 0; r < prefetch_rows; ++r)
+        if(nt * r + tid < b_count)
+          starts[1 + nt * r + tid] = relative(ahead.starts[r]);
+      preceding = ahead.preceding;
+    } else {
+      for(int j = tid; j < b_count; j += nt)
+        starts[1 + j] = relative((int)segments[range.b_begin + j]);
+      if(nt - 1 == tid && range.b_begin)
+        preceding = (int)segments[range.b_begin - 1];
+    }
+    if(nt - 1 == tid) {
+      starts[0] = 0;
+      storage.open_offset = range.b_begin ? range.a_begin - preceding : 0;
+    }
+    __syncthreads();
+    int open_offset = storage.open_offset;
+
+    // 3. one marker per segment that owns items here (see fill()).
+    for(int j = tid; j < b_count; j += nt) {
+      int s0 = starts[1 + j];
+      int s1 = (j + 1 < b_count) ? (int)starts[2 + j] : 0x10000;
+      if(s0 != s1 && s0 < a_count)
+        slots[layout_t::index(s0)] = (slot_t)(j + 1);
+    }
+    __syncthreads();
+
+    // 4. running maximum along the items.
+    scan_compact(tid, a_count, slots, storage.scan);
+    return compact_tile_t { slots, starts, open_offset };
+  }
+
+  MGPU_DEVICE static void scan_compact(int tid, int a_count, slot_t* slots,
+    typename scan_t::storage_t& scan_storage) {
+    int x[vt];
+    PRAGMA_UNROLL
+    for(int c = 0; c < chunks; ++c) {
+      slot_t chunk[W];
+      detail::lds_load_chunk<W>(
+        slots + layout_t::index(vt * tid + W * c), chunk);
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) x[W * c + e] = chunk[e];
+    }
+    PRAGMA_UNROLL
+    for(int i = 1; i < vt; ++i) x[i] = max(x[i - 1], x[i]);
+
+    scan_result_t<int> carry = scan_t().scan(tid, x[vt - 1], scan_storage,
+      nt, maximum_t<int>(), 0, scan_type_exc);
+
+    PRAGMA_UNROLL
+    for(int c = 0; c < chunks; ++c) {
+      slot_t chunk[W];
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e)
+        chunk[e] = (slot_t)max(carry.scan, x[W * c + e]);
+      // Slots at or past a_count belong to the segment starts: leave them.
+      if(vt * tid + W * c < a_count)
+        detail::lds_store_chunk<W>(
+          slots + layout_t::index(vt * tid + W * c), chunk);
+    }
+    __syncthreads();
+  }
+
+  //////////////////////////////////////////////////////////////////////////////
   // Decoding a tile from coarse splits (detail::lbs_block_partition_f): the
   // partition kernel only says in which block of lbs_block starts each of the
   // tile's two splits lies.  The tile loads the starts of those blocks and of
@@ -794,8 +918,21 @@ struct cached_segment_load_t {
   enum { size = tuple_size<pointers_t>::value };
   typedef tuple_iterator_value_t<pointers_t> value_t;
 
+  // Values of up to 8 bytes are staged for up to 2 * nt - 32 segments (two
+  // reads per thread), wider ones for up to nt: a tile of 512 x 16 elements
+  // can begin 873 segments on the 2^24-segment benchmark input, and a tile
+  // with more segments than are staged has every item gather its own value
+  // from global memory, which costs several times what staging does.
+  enum {
+    rows = sizeof(value_t) <= 8 ? 2 : 1,
+    capacity = rows * nt - (rows > 1 ? 32 : 0)
+  };
   struct storage_t {
-    value_t data[nt];
+    value_t data[capacity];
+  };
+  // What fetch() leaves in registers for commit().
+  struct fetched_t {
+    value_t x[rows];
   };
 
   // Stages the values of segments [begin, begin + count) in LDS if they fit
@@ -803,25 +940,34 @@ struct cached_segment_load_t {
   // `count` must be the same in every thread.
   MGPU_DEVICE static bool stage(int tid, int begin, int count,
     storage_t& storage, pointers_t iterators) {
-    value_t x;
+    fetched_t x;
     bool fits = fetch(tid, begin, count, iterators, x);
     commit(tid, begin, count, x, storage);
     return fits;
   }
   // The same in two steps, so that the global read can be in flight while
   // the caller does something else (decodes the tile, say): fetch() issues
-  // the read into a register, commit() puts it into LDS and ends with a
+  // the reads into registers, commit() puts them into LDS and ends with a
   // barrier if the values fit.
   MGPU_DEVICE static bool fetch(int tid, int begin, int count,
-    pointers_t iterators, value_t& x) {
-    if(count > nt) return false;
-    if(tid < count && begin + tid >= 0) x = mgpu::load(iterators, begin + tid);
+    pointers_t iterators, fetched_t& fetched) {
+    if(count > capacity) return false;
+    PRAGMA_UNROLL
+    for(int r = 0; r < rows; ++r) {
+      int at = nt * r + tid;
+      if(at < count && begin + at >= 0)
+        fetched.x[r] = mgpu::load(iterators, begin + at);
+    }
     return true;
   }
   MGPU_DEVICE static void commit(int tid, int begin, int count,
-    const value_t& x, storage_t& storage) {
-    if(count > nt) return;
-    if(tid < count && begin + tid >= 0) storage.data[tid] = x;
+    const fetched_t& fetched, storage_t& storage) {
+    if(count > capacity) return;
+    PRAGMA_UNROLL
+    for(int r = 0; r < rows; ++r) {
+      int at = nt * r + tid;
+      if(at < count && begin + at >= 0) storage.data[at] = fetched.x[r];
+    }
     __syncthreads();
   }
   // Value of segment seg = begin + rel.
@@ -892,14 +1038,16 @@ template<int nt>
 struct cached_segment_load_t<nt, tuple<> > {
   typedef empty_t storage_t;
   typedef tuple<> value_t;
+  typedef empty_t fetched_t;
 
   MGPU_DEVICE static bool stage(int, int, int, storage_t&, tuple<>) {
     return false;
   }
-  MGPU_DEVICE static bool fetch(int, int, int, tuple<>, value_t&) {
+  MGPU_DEVICE static bool fetch(int, int, int, tuple<>, fetched_t&) {
     return false;
   }
-  MGPU_DEVICE static void commit(int, int, int, const value_t&, storage_t&) {
+  MGPU_DEVICE static void commit(int, int, int, const fetched_t&,
+    storage_t&) {
   }
   MGPU_DEVICE static value_t get(bool, int, int, const storage_t&, tuple<>) {
     return value_t();

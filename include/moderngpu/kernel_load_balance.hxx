@@ -19,12 +19,14 @@ BEGIN_MGPU_NAMESPACE
 namespace detail {
 
 // Default tiles for the search on gfx950: 512 threads (two wavefronts per
-// SIMD) x 12 items, 24 KB of item slots per CTA, when the functor takes
-// per-segment cached values; x 16 items when it does not (fewer tiles, so
-// fewer waits for a tile's segment starts: 204 against 216 us for 2^28 items
-// in 2^24 segments, while with cached values 16 items per thread measured
-// 322 against 260 us).
-typedef launch_box_t<arch_gfx950_cta<512, 12, 12> > lbs_launch_default_t;
+// SIMD) x 16 items, with or without per-segment cached values.  On 2^28 items
+// in 2^24 segments: the search 204 us against 216 us with 512 x 12 (fewer
+// tiles, so fewer reads of a tile's segment starts in between the stores);
+// interval_expand 228 against 245 us in its tile kernel.  (Tiles of 512 x 16
+// begin up to 873 segments on that input; while at most 512 segments' values
+// could be staged in LDS a third of the tiles fell back to gathering a value
+// per item and this shape measured 322 us.)
+typedef launch_box_t<arch_gfx950_cta<512, 16, 16> > lbs_launch_default_t;
 typedef launch_box_t<arch_gfx950_cta<512, 16, 16> > lbs_launch_plain_t;
 template<typename pointers_t>
 struct lbs_launch_select_t {
@@ -51,11 +53,12 @@ struct is_chunk_functor_t<func_t,
 //   enum { lbs_tiles_per_cta = 2 };
 // Such a CTA issues the reads of every tile's segment starts and cached
 // values before it works on the first tile, so that the later tiles' have
-// landed when their turn comes.  That pays where a tile is nothing but two
-// dependent reads followed by a stream of stores -- interval_expand: 312 ->
-// 298 us on 2^28 items in 2^24 segments -- and costs elsewhere (the search
-// without cached values 241 -> 250 us, interval_scatter 806 -> 823 us,
-// interval_move 643 -> 685 us), so the default is one tile per CTA.
+// landed when their turn comes.  That pays where a tile is nothing but its
+// reads followed by a stream of stores -- interval_expand: 240 -> 228 us in
+// the tile kernel on 2^28 items in 2^24 segments, the search over coarse
+// splits 217 -> 201 us -- and not where the functor reads or writes scattered
+// memory of its own (interval_scatter 806 -> 823 us, interval_move 643 ->
+// 685 us), so the default is one tile per CTA.
 template<typename func_t, typename enable_t = void>
 struct lbs_tiles_per_cta_t {
   enum { value = 1 };
@@ -97,7 +100,7 @@ struct transform_lbs_f {
     enum { W = load_balance_t::W, chunks = vt / W };
 
     __shared__ struct {
-      typename load_balance_t::storage_t lbs;
+      typename load_balance_t::compact_storage_t lbs;
       typename cached_load_t::storage_t cached;
     } shared;
 
@@ -106,7 +109,7 @@ struct transform_lbs_f {
     // fanned out through LDS when they fit), all issued before anything waits.
     merge_range_t ranges[tiles_per_cta];
     typename load_balance_t::prefetch_t ahead[tiles_per_cta];
-    value_t fetched[tiles_per_cta];
+    typename cached_load_t::fetched_t fetched[tiles_per_cta];
     bool staged[tiles_per_cta];
     PRAGMA_UNROLL
     for(int g = 0; g < tiles_per_cta; ++g) {
@@ -125,16 +128,17 @@ struct transform_lbs_f {
       if(tiles_per_cta * group + g >= num_tiles) break;
       if(g) __syncthreads();            // the previous tile is done with LDS
 
-      // After fill(), LDS slot p holds (segment of tile item p) - seg_base and
-      // the tile's segment starts sit behind the slots.
+      // After fill_compact(), LDS slot p holds (segment of tile item p) -
+      // seg_base, and tile.rank(p, that) is the item's rank in its segment.
       merge_range_t range = ranges[g];
       int a_count = range.a_count();
       int seg_base = range.b_begin - 1;
-      load_balance_t().fill(range, segments, tid, shared.lbs, ahead[g]);
+      typename load_balance_t::compact_tile_t tile =
+        load_balance_t().fill_compact(range, segments, tid, shared.lbs,
+          ahead[g]);
       cached_load_t::commit(tid, seg_base, range.b_count() + 1, fetched[g],
         shared.cached);
-      const int* slots = shared.lbs.indices;
-      const int* starts = slots + load_balance_t::starts_offset(a_count);
+      const typename load_balance_t::slot_t* slots = tile.slots;
 
       // The emission loop exists twice -- cached values staged in LDS, or
       // gathered from global memory -- so that each copy is straight-line code.
@@ -144,32 +148,47 @@ struct transform_lbs_f {
           // The functor consumes W consecutive items at a time (one 16-byte
           // store per chunk for 4-byte results).  Chunk nt * i + tid in step i:
           // consecutive lanes own consecutive chunks.
+          // All LDS reads of the thread's chunks come first and none of
+          // them sits behind a branch (a slot past the tile's items reads
+          // something that is never used, clamped so that what is looked up
+          // with it stays inside its array): the compiler issues them back
+          // to back, and only the stores are conditional.
+          typename load_balance_t::slot_t raw[chunks][W];
+          PRAGMA_UNROLL
+          for(int i = 0; i < chunks; ++i)
+            lds_load_chunk<W>(slots + layout_t::index(W * (nt * i + tid)),
+              raw[i]);
+          int b_count = range.b_count();
           PRAGMA_UNROLL
           for(int i = 0; i < chunks; ++i) {
             int p = W * (nt * i + tid);
             int index = range.a_begin + p;
-            if(p + W <= a_count) {
-              int rel[W], seg[W], rank[W];
-              value_t cached[W];
-              lds_load_chunk<W>(slots + layout_t::index(p), rel);
-              PRAGMA_UNROLL
-              for(int e = 0; e < W; ++e) {
-                seg[e] = seg_base + rel[e];
-                rank[e] = index + e - starts[rel[e]];
-                cached[e] = cached_load_t::get(in_lds, rel[e], seg[e],
+            int rel[W], seg[W], rank[W];
+            value_t cached[W];
+            PRAGMA_UNROLL
+            for(int e = 0; e < W; ++e) {
+              rel[e] = min((int)raw[i][e], b_count);
+              seg[e] = seg_base + rel[e];
+              rank[e] = tile.rank(p + e, rel[e]);
+              if constexpr(in_lds)
+                cached[e] = cached_load_t::get(true, rel[e], seg[e],
                   shared.cached, caching_iterators);
+            }
+            if(p + W <= a_count) {
+              if constexpr(!in_lds) {
+                PRAGMA_UNROLL
+                for(int e = 0; e < W; ++e)
+                  cached[e] = cached_load_t::get(false, rel[e], seg[e],
+                    shared.cached, caching_iterators);
               }
               f.template chunk<W>(index, seg, rank, cached, args...);
             } else {
               PRAGMA_UNROLL
               for(int e = 0; e < W; ++e) {
-                if(p + e < a_count) {
-                  int rel = slots[layout_t::index(p + e)];
-                  int seg = seg_base + rel;
-                  f(index + e, seg, index + e - starts[rel],
-                    cached_load_t::get(in_lds, rel, seg, shared.cached,
+                if(p + e < a_count)
+                  f(index + e, seg[e], rank[e],
+                    cached_load_t::get(in_lds, rel[e], seg[e], shared.cached,
                       caching_iterators), args...);
-                }
               }
             }
           }
@@ -183,7 +202,7 @@ struct transform_lbs_f {
               int rel = slots[layout_t::index(p)];
               int seg = seg_base + rel;
               int index = range.a_begin + p;
-              f(index, seg, index - starts[rel],
+              f(index, seg, tile.rank(p, rel),
                 cached_load_t::get(in_lds, rel, seg, shared.cached,
                   caching_iterators), args...);
             }
@@ -487,10 +506,7 @@ struct lbs_store_seg_f {
 template<>
 struct lbs_store_seg_f<int*> {
   typedef void chunk_functor_tag;
-#ifndef MGPU_EXP_SEARCH_TILES
-#define MGPU_EXP_SEARCH_TILES 2
-#endif
-  enum { lbs_tiles_per_cta = MGPU_EXP_SEARCH_TILES };
+  enum { lbs_tiles_per_cta = 2 };
   int* output;
   MGPU_DEVICE void operator()(int index, int seg, int, tuple<>) const {
     output[index] = seg;

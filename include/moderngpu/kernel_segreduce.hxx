@@ -319,7 +319,7 @@ struct segreduce_tile_f {
       int a_count = range.a_count();
       int seg_base = range.b_begin - 1;
       // The cached values' read is in flight while the tile is decoded.
-      typename cached_load_t::value_t fetched;
+      typename cached_load_t::fetched_t fetched;
       bool staged = cached_load_t::fetch(tid, seg_base, range.b_count() + 1,
         input.caching_iterators, fetched);
       load_balance_t().fill(range, segments, tid, shared.source.lbs);

@@ -111,7 +111,7 @@ struct workcreate_tile_t {
     // anything waits and land while the tile is decoded.
     typename load_balance_t::prefetch_t ahead =
       load_balance_t::prefetch(range, segments, tid);
-    value_t fetched;
+    typename cached_load_t::fetched_t fetched;
     bool staged = cached_load_t::fetch(tid, range.b_begin - 1,
       range.b_count() + 1, caching_iterators, fetched);
     load_balance_t().fill(range, segments, tid, shared.lbs, ahead);

@@ -4,7 +4,9 @@
 // moderngpu uses (src/moderngpu/tuple.hxx:85-391).
 //
 // Layout: tuple<A, B, C> is a value of A followed by tuple<B, C> (recursive
-// aggregate), which keeps it trivially copyable for kernel arguments.
+// aggregate), which keeps it trivially copyable for kernel arguments.  The
+// empty tuple at the end takes no room (sizeof(tuple<int>) == 4, not 8): the
+// kernels keep one tuple of cached values per segment in LDS.
 #pragma once
 #include <utility>
 #include "meta.hxx"
@@ -62,7 +64,14 @@ template<typename arg_t, typename... args_t>
 struct tuple<arg_t, args_t...> {
   typedef tuple<args_t...> tail_t;
   arg_t head;
-  tail_t tail;
+#if defined(__clang__)
+#pragma clang diagnostic push
+#pragma clang diagnostic ignored "-Wc++20-extensions"
+#endif
+  [[no_unique_address]] tail_t tail;
+#if defined(__clang__)
+#pragma clang diagnostic pop
+#endif
 
   tuple() = default;
   tuple(const tuple&) = default;
