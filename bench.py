@@ -345,6 +345,58 @@ def make_c4_gather_probe(copies):
     return wk
 
 
+def make_store_probe(copies, mapping, read_ints):
+    """Not a kernel of this library: the yardstick for the kernels that are
+    streams of stores (tests/csrc/test_kernels.hip, tk_store_probe).  1 GiB of
+    ints is written by CTAs of 512 threads, each one range of about 7,650 ints
+    whose ends are multiples of 32 (what a tile of the search stores); before
+    that each CTA reads read_ints ints of its own from a second array.
+    mapping: 0 tile = blockIdx, 1 runs of 16 tiles per XCD, 2 eighths."""
+    import ctypes
+    import torch
+    tk = ctypes.CDLL(os.path.join(ROOT, "tests", "csrc", "libmgpu_test_kernels.so"))
+    n = 1 << 28
+    rng = np.random.Generator(np.random.PCG64(1))
+    ends = np.cumsum(7650 + rng.integers(-200, 201, size=n // 7650 + 8))
+    ends = np.unique((ends - ends % 32)[ends < n - 8000])
+    begins = np.concatenate([[0], ends, [n]]).astype(np.int32)
+    tiles = begins.size - 1
+    d_begins = _dev(begins)
+    outs = [torch.empty(n, dtype=torch.int32, device="cuda") for _ in range(min(copies, 2))]
+    source = torch.zeros(max(read_ints, 1) * tiles + 512, dtype=torch.int32, device="cuda")
+    wk = Workload()
+    names = ["tile = blockIdx", "runs of 16 tiles per XCD", "one eighth of the tiles per XCD"]
+    wk.key = "store_probe_%s_read%d" % (["linear", "runs", "eighths"][mapping], read_ints)
+    wk.dtype, wk.items = "i32", n
+    wk.name = ("store yardstick: 1 GiB in %d ragged tiles, %s, %d bytes read per tile"
+               % (tiles, names[mapping], 4 * read_ints))
+    wk.bytes = n * 4 + read_ints * 4 * tiles
+    wk.kernel = "store_probe_k (yardstick, not part of the library)"
+    stream = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+    def step(i):
+        out = outs[i % len(outs)]
+        rc = tk.tk_store_probe(ctypes.c_void_p(out.data_ptr()),
+                               ctypes.c_void_p(d_begins.data_ptr()), tiles, mapping, read_ints,
+                               ctypes.c_void_p(source.data_ptr()), stream())
+        assert rc == 0, rc
+        return out
+    wk.step = wk.tiles = step
+
+    def check():
+        # Every tile is a whole number of groups of four: q, x, 2, 3 with q the
+        # position in the tile and x = 0 (the source array is all zeros).
+        got = step(0)
+        b = d_begins.long()
+        first = torch.arange(n, device="cuda") - torch.repeat_interleave(b[:-1], b[1:] - b[:-1])
+        m = first % 4
+        want = torch.where(m == 0, first, torch.where(m == 1, torch.zeros_like(m), m)).int()
+        return bool(torch.equal(got, want))
+    wk.check = check
+    wk.cpu = lambda: (lambda: np.zeros(n, dtype=np.int32))
+    return wk
+
+
 def make_c5(copies, kind):
     import torch
     import moderngpu_amd as m
@@ -522,6 +574,13 @@ FACTORIES = {
     "inner_join_i32": lambda c: make_search(c, "join"),
     "c4_spmv_f32": make_c4,
     "c4_gather_probe_f32": make_c4_gather_probe,
+    "store_probe_linear_read0": lambda c: make_store_probe(c, 0, 0),
+    "store_probe_runs_read0": lambda c: make_store_probe(c, 1, 0),
+    "store_probe_eighths_read0": lambda c: make_store_probe(c, 2, 0),
+    "store_probe_linear_read512": lambda c: make_store_probe(c, 0, 512),
+    "store_probe_runs_read512": lambda c: make_store_probe(c, 1, 512),
+    "store_probe_eighths_read512": lambda c: make_store_probe(c, 2, 512),
+    "store_probe_eighths_read64": lambda c: make_store_probe(c, 2, 64),
     "c5_f64max": lambda c: make_c5(c, "f64max"),
     "c5_i64sum": lambda c: make_c5(c, "i64sum"),
 }

@@ -297,3 +297,57 @@ API int tk_load_balance(int nt, int vt, int count, const int* segments,
 #undef LB
   return -1;
 }
+
+////////////////////////////////////////////////////////////////////////////////
+// A yardstick for the kernels that are streams of stores (the load-balancing
+// search family): CTA `tile` stores the ints [begins[tile], begins[tile + 1])
+// with 16-byte stores, after reading read_ints ints of `source` (from
+// read_ints * tile on; read_ints <= 512) that the stored values depend on.
+// mapping: 0 tile = blockIdx, 1 runs of 16 tiles per XCD (xcd_tile),
+// 2 one contiguous eighth of the tiles per XCD (xcd_tile_eighths).
+// The grid is xcd_grid(num_tiles).  Launches on `stream` and does not wait.
+
+namespace {
+template<int mapping>
+__global__ __launch_bounds__(512) void store_probe_k(int* out,
+  const int* begins, int num_tiles, int read_ints, const int* source) {
+  int tile = 0 == mapping ? (int)blockIdx.x :
+    1 == mapping ? detail::xcd_tile(blockIdx.x, num_tiles) :
+    detail::xcd_tile_eighths(blockIdx.x, num_tiles);
+  if(tile >= num_tiles) return;
+  __shared__ int exchange[512];
+  int tid = threadIdx.x;
+  int x = tid < read_ints ? source[(size_t)read_ints * tile + tid] : 0;
+  exchange[tid] = x;
+  __syncthreads();
+  x = exchange[(tid + 1) % 512];
+  int begin = begins[tile], n = begins[tile + 1] - begin;
+  typedef int v4_t __attribute__((ext_vector_type(4), aligned(4)));
+  for(int q = 4 * tid; q < n; q += 4 * 512) {
+    if(q + 4 <= n) {
+      v4_t v = { q, x, 2, 3 };
+      *(v4_t*)(out + begin + q) = v;
+    } else
+      for(int e = 0; e < 4; ++e)
+        if(q + e < n) out[begin + q + e] = x;
+  }
+}
+} // namespace
+
+API int tk_store_probe(int* out, const int* begins, int num_tiles,
+  int mapping, int read_ints, const int* source, void* stream) {
+  if(num_tiles <= 0 || read_ints < 0 || read_ints > 512 ||
+    mapping < 0 || mapping > 2)
+    return (int)hipErrorInvalidValue;
+  int grid = detail::xcd_grid(num_tiles);
+  hipStream_t s = (hipStream_t)stream;
+  switch(mapping) {
+    case 0: hipLaunchKernelGGL(store_probe_k<0>, dim3(grid), dim3(512), 0, s,
+      out, begins, num_tiles, read_ints, source); break;
+    case 1: hipLaunchKernelGGL(store_probe_k<1>, dim3(grid), dim3(512), 0, s,
+      out, begins, num_tiles, read_ints, source); break;
+    default: hipLaunchKernelGGL(store_probe_k<2>, dim3(grid), dim3(512), 0, s,
+      out, begins, num_tiles, read_ints, source); break;
+  }
+  return (int)hipGetLastError();
+}
