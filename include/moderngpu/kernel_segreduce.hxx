@@ -26,7 +26,7 @@
 //       The segment that was already open when the tile began is reported as
 //       a (segment, partial) carry for the spine.
 //   K3  segreduce_spine_f folds the per-tile carries of segments that span
-//       tiles into output[] in one launch (1024 carries per CTA; a run of
+//       tiles into output[] in one launch (256 carries per CTA; a run of
 //       carries that crosses CTAs is finished by the CTA it ends in).
 // The CUDA reference instead walks vt + 1 merged elements per thread through
 // dependent shared-memory reads and runs a recursive fix-up, one launch per

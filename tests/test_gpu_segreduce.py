@@ -153,7 +153,8 @@ def test_config5_scaled(dev, oracle, kind):
 
 
 def test_spine_levels(dev, oracle):
-    """More than 1024 tiles in one segment forces the second spine level; a
+    """One segment over more than 2,600 tiles: its run of carries crosses ten
+    spine CTAs (256 carries each) and is finished by the CTA it ends in; a
     segment that begins exactly on a tile edge takes the overwrite path."""
     import moderngpu_amd as m
     rng = np.random.default_rng(23)
