@@ -178,3 +178,43 @@ def test_config3_full_size_properties(dev):
     vals = _dev(w["values"])
     exp = m.interval_expand(vals, count, segs)
     assert torch.equal(exp, vals[got.long()])
+
+
+def test_memory_properties_and_store_yardstick(dev):
+    """mgpu_hip_memory_properties returns what hipDeviceProp_t holds; the store
+    yardstick of the test kernels writes every int of its ranges under each of
+    its three tile-to-CTA mappings, with and without the read in front."""
+    import ctypes
+    import torch
+    import moderngpu_amd as m
+    clock, width = ctypes.c_int(0), ctypes.c_int(0)
+    assert m.lib().mgpu_hip_memory_properties(0, ctypes.addressof(clock),
+                                              ctypes.addressof(width)) == 0
+    assert clock.value > 0 and width.value > 0 and width.value % 64 == 0
+    assert m.lib().mgpu_hip_memory_properties(0, None, None) == 1      # hipErrorInvalidValue
+
+    tk = ctypes.CDLL(os.path.join(os.path.dirname(__file__), "csrc", "libmgpu_test_kernels.so"))
+    rng = np.random.default_rng(5)
+    lengths = 32 * rng.integers(1, 300, size=333)
+    begins = np.concatenate([[0], np.cumsum(lengths)]).astype(np.int32)
+    n, tiles = int(begins[-1]), lengths.size
+    d_begins = _dev(begins)
+    source = torch.arange(512 * tiles, dtype=torch.int32, device="cuda")
+    pos = np.arange(n) - np.repeat(begins[:-1], lengths)
+    tile_of = np.repeat(np.arange(tiles), lengths)
+    for mapping in (0, 1, 2):
+        for read_ints in (0, 64, 512):
+            out = torch.full((n + 8,), -1, dtype=torch.int32, device="cuda")
+            assert tk.tk_store_probe(ctypes.c_void_p(out.data_ptr()),
+                                     ctypes.c_void_p(d_begins.data_ptr()), tiles, mapping,
+                                     read_ints, ctypes.c_void_p(source.data_ptr()), None) == 0
+            torch.cuda.synchronize()
+            got = out.cpu().numpy()
+            assert (got[n:] == -1).all()
+            # groups of four: position in the tile, x, 2, 3, where x is what the
+            # thread's right-hand neighbour read (0 beyond read_ints)
+            thread = (pos // 4) % 512
+            neighbour = (thread + 1) % 512
+            x = np.where(neighbour < read_ints, read_ints * tile_of + neighbour, 0)
+            want = np.select([pos % 4 == 0, pos % 4 == 1], [pos, x], pos % 4)
+            assert np.array_equal(got[:n], want), (mapping, read_ints)

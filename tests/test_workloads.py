@@ -57,3 +57,23 @@ def test_config5_small():
         ln = _lengths(d["segments"], n)
         assert ln.sum() == n and _valid(d["segments"], n)
         assert (ln > n // 8).sum() == 4 and set(np.unique(ln[ln <= n // 8])) <= {0, 1}
+
+
+def test_disk_cache_returns_the_same_arrays(tmp_path, monkeypatch):
+    """With MGPU_WORKLOAD_CACHE set a configuration is generated once, kept as
+    .npz, and read back with the same values and types (profiler runs use
+    this to start several runs of one workload quickly)."""
+    monkeypatch.setenv("MGPU_WORKLOAD_CACHE", str(tmp_path))
+    first = w.config5(scale=256, kind="i64sum")
+    assert any(p.suffix == ".npz" for p in tmp_path.iterdir())
+    again = w.config5(scale=256, kind="i64sum")
+    assert set(first) == set(again)
+    for key in first:
+        if isinstance(first[key], np.ndarray):
+            assert first[key].dtype == again[key].dtype
+            assert np.array_equal(first[key], again[key])
+        else:
+            assert first[key] == again[key] and type(first[key]) is type(again[key])
+    monkeypatch.delenv("MGPU_WORKLOAD_CACHE")
+    plain = w.config5(scale=256, kind="i64sum")
+    assert np.array_equal(plain["values"], first["values"])
