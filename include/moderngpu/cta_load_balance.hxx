@@ -141,10 +141,7 @@ enum { lbs_snap_items = 32, lbs_snap_window = 32, lbs_snap_slack = 64 };
 
 // Segment starts per block of the coarse partition (lbs_block_partition_f in
 // search.hxx, cta_load_balance_t::fill_blocks below).
-#ifndef MGPU_LBS_BLOCK
-#define MGPU_LBS_BLOCK 256
-#endif
-enum { lbs_block = MGPU_LBS_BLOCK };
+enum { lbs_block = 256 };
 
 MGPU_HOST_DEVICE constexpr int lbs_tile_spacing(int nv) {
   return nv >= 8 * lbs_snap_slack ? nv - lbs_snap_slack : nv;
@@ -976,40 +973,6 @@ struct cached_segment_load_t {
     return staged ? storage.data[rel] : mgpu::load(iterators, max(seg, 0));
   }
 
-  // For tiles decoded from coarse splits (cta_load_balance_t::fill_blocks):
-  // the values of the segments whose starts the tile loads, held in LDS at
-  // (segment - first loaded segment) when there are at most block_capacity
-  // of them.  fetch4() reads the values of four consecutive segments from j
-  // on (those below end) into registers, stage4() puts them at 4 * q ... in
-  // LDS (the caller places the barrier).
-  enum { block_capacity = sizeof(value_t) <= 8 ? 2 * nt : nt };
-  struct block_storage_t {
-    alignas(16) value_t data[block_capacity];
-  };
-  MGPU_DEVICE static void fetch4(int j, int end, pointers_t iterators,
-    value_t (&x)[4]) {
-    if(j + 4 <= end) {
-      PRAGMA_UNROLL
-      for(int e = 0; e < 4; ++e) x[e] = mgpu::load(iterators, j + e);
-    } else {
-      PRAGMA_UNROLL
-      for(int e = 0; e < 4; ++e)
-        if(j + e < end) x[e] = mgpu::load(iterators, j + e);
-    }
-  }
-  MGPU_DEVICE static void stage4(int q, int count, const value_t (&x)[4],
-    block_storage_t& storage) {
-    if(4 * q < count && 4 * q + 4 <= block_capacity) {
-      PRAGMA_UNROLL
-      for(int e = 0; e < 4; ++e) storage.data[4 * q + e] = x[e];
-    }
-  }
-  MGPU_DEVICE static value_t get_block(bool staged, int at, int seg,
-    const block_storage_t& storage, pointers_t iterators) {
-    return staged ? storage.data[max(at, 0)] :
-      mgpu::load(iterators, max(seg, 0));
-  }
-
   // range = segments the tile's items can belong to.
   template<int vt0, int vt>
   MGPU_DEVICE static array_t<value_t, vt> load(int tid, int count,
@@ -1052,16 +1015,6 @@ struct cached_segment_load_t<nt, tuple<> > {
   MGPU_DEVICE static value_t get(bool, int, int, const storage_t&, tuple<>) {
     return value_t();
   }
-  enum { block_capacity = 0 };
-  typedef empty_t block_storage_t;
-  MGPU_DEVICE static void fetch4(int, int, tuple<>, value_t (&)[4]) { }
-  MGPU_DEVICE static void stage4(int, int, const value_t (&)[4],
-    block_storage_t&) { }
-  MGPU_DEVICE static value_t get_block(bool, int, int,
-    const block_storage_t&, tuple<>) {
-    return value_t();
-  }
-
   template<int vt0, int vt>
   MGPU_DEVICE static array_t<value_t, vt> load(int, int, range_t,
     array_t<int, vt>, storage_t&, tuple<>) {

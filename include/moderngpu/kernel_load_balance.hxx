@@ -215,22 +215,22 @@ struct transform_lbs_f {
   }
 };
 
-// The same tile kernel over coarse splits (load_balance_block_partitions):
-// mp_data[tile] is the block of lbs_block segment starts in which the tile's
-// first split falls.  The tile reads the starts of its two blocks and of what
-// lies between them and finds its exact (and snapped) splits itself
-// (cta_load_balance_t::fill_blocks), so the partition kernel reads one start
-// in lbs_block instead of all of them: 6 instead of 24 us for 2^24 starts.
-// The tile reads up to a block of starts more at either end than its own, and
-// so it does with the cached values.
+// The tile kernel over coarse splits (load_balance_block_partitions), for
+// functors without cached values: mp_data[tile] is the block of lbs_block
+// segment starts in which the tile's first split falls.  The tile reads the
+// starts of its two blocks and of what lies between them and finds its exact
+// (and snapped) splits itself (cta_load_balance_t::fill_blocks), so the
+// partition kernel reads one start in lbs_block instead of all of them: 6
+// instead of 24 us for 2^24 starts.  The starts a tile reads beyond its own
+// (up to a block at either end) mostly come from the L2: the tiles next to
+// it, which own them, run on the same XCD.
 template<typename launch_t, typename func_t, typename segments_it,
-  typename pointers_t, typename int_t>
+  typename int_t>
 struct transform_lbs_blocks_f {
   func_t f;
   int count;
   segments_it segments;
   int num_segments;
-  pointers_t caching_iterators;
   const int_t* mp_data;
   int num_tiles;
 
@@ -249,37 +249,22 @@ struct transform_lbs_blocks_f {
     enum { nt = params_t::nt, vt = params_t::vt };
     typedef cta_load_balance_t<nt, vt> load_balance_t;
     typedef typename load_balance_t::layout_t layout_t;
-    typedef cached_segment_load_t<nt, pointers_t> cached_load_t;
-    typedef typename cached_load_t::value_t value_t;
     enum { W = load_balance_t::W, chunks = vt / W };
-
-    enum { rows = load_balance_t::block_rows };
     constexpr int spacing = lbs_tile_spacing(load_balance_t::nv);
     constexpr bool snap = spacing < load_balance_t::nv;
 
-    __shared__ struct {
-      typename load_balance_t::block_storage_t lbs;
-      typename cached_load_t::block_storage_t cached;
-    } shared;
+    __shared__ typename load_balance_t::block_storage_t shared;
 
     // Which starts each tile has to load (its own and up to a block at either
-    // end, see cta_load_balance_t::fill_blocks), with the reads of the starts
-    // and of the same segments' cached values issued before anything waits.
+    // end, see cta_load_balance_t::fill_blocks), with the reads issued before
+    // anything waits.
     typename load_balance_t::block_tile_t ahead[tiles_per_cta];
-    value_t fetched[tiles_per_cta][rows][4];
     PRAGMA_UNROLL
     for(int g = 0; g < tiles_per_cta; ++g) {
       int tile = tiles_per_cta * group + g;
-      if(tile < num_tiles) {
+      if(tile < num_tiles)
         ahead[g] = load_balance_t::block_prefetch(count, num_segments, tile,
           spacing, mp_data, segments, tid);
-        if(ahead[g].ahead) {
-          PRAGMA_UNROLL
-          for(int r = 0; r < rows; ++r)
-            cached_load_t::fetch4(ahead[g].jb + 4 * (nt * r + tid),
-              ahead[g].je, caching_iterators, fetched[g][r]);
-        }
-      }
     }
 
     PRAGMA_UNROLL
@@ -289,82 +274,55 @@ struct transform_lbs_blocks_f {
 
       // After fill_blocks(), LDS slot p holds (segment of tile item p) -
       // seg_base and starts[rel] is the start of segment seg_base + rel.
-      // The cached values of all the segments whose starts were loaded go to
-      // LDS too when they fit, at (segment - first loaded segment).
-      bool staged = 0 != tuple_size<pointers_t>::value && ahead[g].ahead &&
-        ahead[g].je - ahead[g].jb <= (int)cached_load_t::block_capacity;
       const int* starts;
       merge_range_t range = load_balance_t::fill_blocks(ahead[g], count,
-        num_segments, segments, snap, tid, shared.lbs, starts, [&]() {
-          if(staged) {
-            PRAGMA_UNROLL
-            for(int r = 0; r < rows; ++r)
-              cached_load_t::stage4(nt * r + tid,
-                ahead[g].je - ahead[g].jb, fetched[g][r], shared.cached);
-          }
-        });
+        num_segments, segments, snap, tid, shared, starts);
       int a_count = range.a_count();
       int seg_base = range.b_begin - 1;
-      int cached_base = seg_base - ahead[g].jb;
-      const int* slots = shared.lbs.indices;
+      const int* slots = shared.indices;
 
-      // The emission loop exists twice -- cached values staged in LDS, or
-      // gathered from global memory -- so that each copy is straight-line code.
-      auto emit_all = [&](auto staged_tag) {
-        constexpr bool in_lds = decltype(staged_tag)::value;
-        if constexpr(is_chunk_functor_t<func_t>::value) {
-          // The functor consumes W consecutive items at a time (one 16-byte
-          // store per chunk for 4-byte results).  Chunk nt * i + tid in step i:
-          // consecutive lanes own consecutive chunks.
-          PRAGMA_UNROLL
-          for(int i = 0; i < chunks; ++i) {
-            int p = W * (nt * i + tid);
-            int index = range.a_begin + p;
-            if(p + W <= a_count) {
-              int rel[W], seg[W], rank[W];
-              value_t cached[W];
-              lds_load_chunk<W>(slots + layout_t::index(p), rel);
-              PRAGMA_UNROLL
-              for(int e = 0; e < W; ++e) {
-                seg[e] = seg_base + rel[e];
-                rank[e] = index + e - starts[rel[e]];
-                cached[e] = cached_load_t::get_block(in_lds,
-                  cached_base + rel[e], seg[e], shared.cached,
-                  caching_iterators);
-              }
-              f.template chunk<W>(index, seg, rank, cached, args...);
-            } else {
-              PRAGMA_UNROLL
-              for(int e = 0; e < W; ++e) {
-                if(p + e < a_count) {
-                  int rel = slots[layout_t::index(p + e)];
-                  int seg = seg_base + rel;
-                  f(index + e, seg, index + e - starts[rel],
-                    cached_load_t::get_block(in_lds, cached_base + rel, seg,
-                      shared.cached, caching_iterators), args...);
-                }
-              }
+      if constexpr(is_chunk_functor_t<func_t>::value) {
+        // The functor consumes W consecutive items at a time (one 16-byte
+        // store per chunk for 4-byte results).  Chunk nt * i + tid in step i:
+        // consecutive lanes own consecutive chunks.
+        PRAGMA_UNROLL
+        for(int i = 0; i < chunks; ++i) {
+          int p = W * (nt * i + tid);
+          int index = range.a_begin + p;
+          if(p + W <= a_count) {
+            int rel[W], seg[W], rank[W];
+            tuple<> cached[W];
+            lds_load_chunk<W>(slots + layout_t::index(p), rel);
+            PRAGMA_UNROLL
+            for(int e = 0; e < W; ++e) {
+              seg[e] = seg_base + rel[e];
+              rank[e] = index + e - starts[rel[e]];
             }
-          }
-        } else {
-          // One item per call, item nt * i + tid in step i: whatever the
-          // functor stores per item is coalesced across the wavefront.
-          PRAGMA_UNROLL
-          for(int i = 0; i < vt; ++i) {
-            int p = nt * i + tid;
-            if(p < a_count) {
-              int rel = slots[layout_t::index(p)];
-              int seg = seg_base + rel;
-              int index = range.a_begin + p;
-              f(index, seg, index - starts[rel],
-                cached_load_t::get_block(in_lds, cached_base + rel, seg,
-                  shared.cached, caching_iterators), args...);
+            f.template chunk<W>(index, seg, rank, cached, args...);
+          } else {
+            PRAGMA_UNROLL
+            for(int e = 0; e < W; ++e) {
+              if(p + e < a_count) {
+                int rel = slots[layout_t::index(p + e)];
+                f(index + e, seg_base + rel, index + e - starts[rel],
+                  tuple<>(), args...);
+              }
             }
           }
         }
-      };
-      if(staged) emit_all(std::true_type());
-      else emit_all(std::false_type());
+      } else {
+        // One item per call, item nt * i + tid in step i: whatever the
+        // functor stores per item is coalesced across the wavefront.
+        PRAGMA_UNROLL
+        for(int i = 0; i < vt; ++i) {
+          int p = nt * i + tid;
+          if(p < a_count) {
+            int rel = slots[layout_t::index(p)];
+            int index = range.a_begin + p;
+            f(index, seg_base + rel, index - starts[rel], tuple<>(), args...);
+          }
+        }
+      }
     }
   }
 };
@@ -374,18 +332,16 @@ struct transform_lbs_blocks_f {
 namespace detail {
 
 // Which of the two tile kernels a call uses.  Without cached values the tiles
-// work from coarse splits (2^28 items in 2^24 segments: 209 against 233 us
-// for the call).  With cached values they keep exact splits: a tile that
-// reads a block of starts more at either end reads that many more values too,
-// which costs more than the cheaper partition kernel saves (interval_expand
-// 297 against 279 us, interval_move 731 against 638 us on the same input).
-#ifndef MGPU_LBS_COARSE_CACHED
-#define MGPU_LBS_COARSE_CACHED 0
-#endif
+// work from coarse splits (2^28 items in 2^24 segments: 210 against 233 us
+// for the call).  With cached values they keep exact splits: the same decode
+// for them took the same time in the tile kernel, but the partition kernel
+// over exact splits streams all the starts right before the tile kernel and
+// leaves them in the memory-side cache, and without that the tile kernel
+// loses what the cheaper partition saves (interval_expand 257 against 256 us
+// as a call, interval_move 647 against 631 us).
 template<typename pointers_t>
 struct lbs_coarse_splits_t {
-  enum { value = MGPU_LBS_COARSE_CACHED ||
-    0 == tuple_size<pointers_t>::value };
+  enum { value = 0 == tuple_size<pointers_t>::value };
 };
 
 // count + num_segments as the 32-bit total the kernels index with; throws
@@ -441,9 +397,8 @@ void transform_lbs_launch(func_t f, int count, segments_it segments,
       load_balance_block_partitions(count, segments, num_segments,
         lbs_tile_spacing(nv), mp_data, context);
     if(phases & lbs_phase_tiles) {
-      transform_lbs_blocks_f<launch_t, func_t, segments_it, pointers_t, int>
-        k { f, count, segments, num_segments, caching_iterators, mp_data,
-          num_tiles };
+      transform_lbs_blocks_f<launch_t, func_t, segments_it, int>
+        k { f, count, segments, num_segments, mp_data, num_tiles };
       cta_launch<launch_t>(k, xcd_grid(k.num_ctas(num_tiles)), context,
         args...);
     }
