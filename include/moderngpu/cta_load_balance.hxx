@@ -522,7 +522,6 @@ struct cta_load_balance_t {
   // per CTA, with 512 x 16 tiles 19 KB instead of 37 KB.
 
   typedef unsigned short slot_t;
-  static_assert(nv + 2 < 65536, "16-bit tile slots need tiles below 2^16");
 
   struct compact_storage_t {
     // Item slots (padded layout), then the relative starts: entry 0 is zero
@@ -548,6 +547,7 @@ struct cta_load_balance_t {
   MGPU_DEVICE compact_tile_t fill_compact(merge_range_t range,
     segments_it segments, int tid, compact_storage_t& storage,
     prefetch_t ahead) const {
+    static_assert(nv + 2 < 65536, "16-bit tile slots need tiles below 2^16");
 
     int a_count = range.a_count();
     int b_count = range.b_count();
