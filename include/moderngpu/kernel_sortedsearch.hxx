@@ -118,20 +118,122 @@ struct sorted_search_f {
   }
 };
 
+// The tile splits of a large search, found in two steps.  A scalar binary
+// search per split over 2^26 + 2^26 keys is 27 dependent pairs of scattered
+// reads, of which the first ten or so find their cache lines in the L2 (every
+// split's search starts at the same places) and the rest do not: 48 us for
+// 43,700 splits, a quarter of the whole call, with the device all but idle.
+// Here every search_sample-th key of both inputs is first copied into two
+// small arrays (2 x 64 K keys for 2^26: they stay in the L2), the search
+// runs over those as far as they go -- needle positions g k + g - 1 pair
+// with haystack positions that are multiples of g when the cross-diagonal
+// is one, which the diagonals of the tiles are -- and only the last
+// log2(search_sample) steps touch the inputs themselves, within one window of
+// search_sample keys of each.
+enum { search_sample = 1024, search_sample_min_total = 1 << 22 };
+
+// Keys of sample storage sorted_search_launch needs (0: no sampling).
+MGPU_HOST_DEVICE size_t sorted_search_sample_count(int64_t num_needles,
+  int64_t num_haystack, int nv) {
+  if(nv % search_sample || num_needles + num_haystack <
+    search_sample_min_total) return 0;
+  return (size_t)(num_needles / search_sample +
+    div_up(num_haystack, (int64_t)search_sample));
+}
+
+template<typename needles_it, typename haystack_it, typename type_t>
+struct search_sample_f {
+  needles_it needles; haystack_it haystack;
+  int needle_samples;
+  type_t* samples;              // needle samples, then haystack samples
+  MGPU_DEVICE void operator()(int index) const {
+    enum { g = search_sample };
+    samples[index] = index < needle_samples ?
+      (type_t)needles[g * index + g - 1] :
+      (type_t)haystack[g * (index - needle_samples)];
+  }
+};
+
+template<bounds_t bounds, typename needles_it, typename haystack_it,
+  typename type_t, typename comp_t>
+struct sampled_partition_f {
+  needles_it needles; haystack_it haystack;
+  int num_needles, num_haystack, nv;
+  comp_t comp;
+  const type_t* samples;
+  int needle_samples;
+  int* p;
+
+  MGPU_DEVICE bool takes_needle(const type_t& a_key,
+    const type_t& b_key) const {
+    return (bounds_upper == bounds) ? comp(a_key, b_key) :
+      !comp(b_key, a_key);
+  }
+
+  MGPU_DEVICE void operator()(int index) const {
+    enum { g = search_sample };
+    int64_t total = (int64_t)num_needles + num_haystack;
+    int64_t d = (int64_t)nv * index;
+    int diag = (int)(d < total ? d : total);
+    int begin = max(0, diag - num_haystack);
+    int end = min(diag, num_needles);
+
+    if(0 == diag % g) {
+      // Needle positions g k + g - 1 inside [begin, end): k in [k0, k1).
+      int k0 = begin <= g - 1 ? 0 : div_up(begin - (g - 1), (int)g);
+      int k1 = end >= g ? (end - g) / g + 1 : 0;
+      int lo = k0, hi = max(k0, k1);
+      const type_t* hay_samples = samples + needle_samples;
+      while(lo < hi) {
+        int k = (int)(((unsigned)lo + (unsigned)hi) / 2);
+        if(takes_needle(samples[k], hay_samples[diag / g - k - 1]))
+          lo = k + 1;
+        else hi = k;
+      }
+      // Position g (lo - 1) + g - 1 takes a needle, g lo + g - 1 does not.
+      if(lo > k0) begin = max(begin, g * lo);
+      if(lo < k1) end = min(end, g * lo + g - 1);
+    }
+    while(begin < end) {
+      int mid = (int)(((unsigned)begin + (unsigned)end) / 2);
+      if(takes_needle(needles[mid], haystack[diag - 1 - mid]))
+        begin = mid + 1;
+      else end = mid;
+    }
+    p[index] = begin;
+  }
+};
+
 // Splits in caller-provided device memory: div_up(num_needles +
-// num_haystack, nv) + 1 ints.
+// num_haystack, nv) + 1 ints, and sorted_search_sample_count() keys (or
+// null: the splits are then found by plain binary searches).
 template<bounds_t bounds, typename launch_t, typename needles_it,
   typename haystack_it, typename indices_it, typename comp_t>
 void sorted_search_launch(needles_it needles, int num_needles,
   haystack_it haystack, int num_haystack, indices_it indices, comp_t comp,
-  int* mp_data, context_t& context) {
+  int* mp_data,
+  typename std::iterator_traits<needles_it>::value_type* samples,
+  context_t& context) {
+  typedef typename std::iterator_traits<needles_it>::value_type type_t;
   int64_t total = (int64_t)num_needles + num_haystack;
   if(total >= ((int64_t)1 << 31)) throw cuda_exception_t(hipErrorInvalidValue);
   if(!num_needles) return;
   int nv = launch_t::nv(context);
   int num_tiles = div_up((int)total, nv);
-  merge_path_partitions_into<bounds>(needles, (int64_t)num_needles, haystack,
-    (int64_t)num_haystack, (int64_t)nv, comp, mp_data, context);
+  size_t num_samples = sorted_search_sample_count(num_needles, num_haystack,
+    nv);
+  if(samples && num_samples) {
+    int needle_samples = num_needles / search_sample;
+    search_sample_f<needles_it, haystack_it, type_t>
+      sample { needles, haystack, needle_samples, samples };
+    transform<256>(sample, num_samples, context);
+    sampled_partition_f<bounds, needles_it, haystack_it, type_t, comp_t>
+      split { needles, haystack, num_needles, num_haystack, nv, comp,
+        samples, needle_samples, mp_data };
+    transform<256>(split, (size_t)num_tiles + 1, context);
+  } else
+    merge_path_partitions_into<bounds>(needles, (int64_t)num_needles,
+      haystack, (int64_t)num_haystack, (int64_t)nv, comp, mp_data, context);
   sorted_search_f<bounds, launch_t, needles_it, haystack_it, indices_it,
     comp_t> k { needles, num_needles, haystack, num_haystack, indices, comp,
       mp_data, num_tiles };
@@ -152,10 +254,14 @@ void sorted_search(needles_it needles, int num_needles, haystack_it haystack,
     needles, num_needles, haystack, num_haystack, indices, comp, context))
     return;
   int64_t total = (int64_t)num_needles + num_haystack;
-  mem_t<int> partitions((size_t)div_up(total, (int64_t)launch_t::nv(context))
-    + 1, context);
+  typedef typename std::iterator_traits<needles_it>::value_type type_t;
+  int nv = launch_t::nv(context);
+  mem_t<int> partitions((size_t)div_up(total, (int64_t)nv) + 1, context);
+  mem_t<type_t> samples(detail::sorted_search_sample_count(num_needles,
+    num_haystack, nv), context);
   detail::sorted_search_launch<bounds, launch_t>(needles, num_needles,
-    haystack, num_haystack, indices, comp, partitions.data(), context);
+    haystack, num_haystack, indices, comp, partitions.data(), samples.data(),
+    context);
 }
 
 END_MGPU_NAMESPACE

@@ -18,11 +18,21 @@ size_t search_partitions(int num_needles, int num_haystack) {
   return (size_t)div_up((int64_t)num_needles + num_haystack,
     (int64_t)search_nv()) + 1;
 }
+size_t search_samples(int num_needles, int num_haystack) {
+  return detail::sorted_search_sample_count(num_needles, num_haystack,
+    search_nv());
+}
+// The splits, then (256-byte aligned) the key samples.
+size_t search_samples_offset(int num_needles, int num_haystack) {
+  return (sizeof(int) * search_partitions(num_needles, num_haystack) + 255) &
+    ~(size_t)255;
+}
 
 // Temporaries of mgpu_hip_inner_join_count, which mgpu_hip_inner_join_pairs
 // reads again.
 struct join_workspace_t {
-  int* lower; int* upper; int* starts; int* partitions; int* partials;
+  int* lower; int* upper; int* starts; int* partitions; int* samples;
+  int* partials;
   size_t bytes;
   join_workspace_t(int a_count, int b_count, void* base) {
     char* at = (char*)base;
@@ -35,6 +45,7 @@ struct join_workspace_t {
     upper = take(a_count);
     starts = take(a_count);
     partitions = take(search_partitions(a_count, b_count));
+    samples = take(search_samples(a_count, b_count));
     partials = take(detail::scan_partials_count(a_count,
       scan_launch_t::sm_ptx::nt * scan_launch_t::sm_ptx::vt));
     bytes = (size_t)(at - (char*)base);
@@ -57,7 +68,8 @@ extern "C" {
 size_t mgpu_hip_sorted_search_workspace_bytes(int num_needles,
   int num_haystack) {
   if(!sizes_ok(num_needles, num_haystack)) return 0;
-  return sizeof(int) * search_partitions(num_needles, num_haystack);
+  return search_samples_offset(num_needles, num_haystack) +
+    sizeof(int) * search_samples(num_needles, num_haystack);
 }
 
 int mgpu_hip_sorted_search(const int* needles, int num_needles,
@@ -71,15 +83,17 @@ int mgpu_hip_sorted_search(const int* needles, int num_needles,
   if(!workspace || workspace_bytes <
     mgpu_hip_sorted_search_workspace_bytes(num_needles, num_haystack))
     return (int)hipErrorInvalidValue;
+  int* samples = (int*)((char*)workspace +
+    search_samples_offset(num_needles, num_haystack));
   return guarded(stream, [&](context_t& context) {
     if(MGPU_BOUNDS_LOWER == bounds)
       detail::sorted_search_launch<bounds_lower, search_launch_t>(needles,
         num_needles, haystack, num_haystack, indices, less_t<int>(),
-        (int*)workspace, context);
+        (int*)workspace, samples, context);
     else
       detail::sorted_search_launch<bounds_upper, search_launch_t>(needles,
         num_needles, haystack, num_haystack, indices, less_t<int>(),
-        (int*)workspace, context);
+        (int*)workspace, samples, context);
   });
 }
 
@@ -98,9 +112,11 @@ int mgpu_hip_inner_join_count(const int* a, int a_count, const int* b,
     return (int)hipErrorInvalidValue;
   return guarded(stream, [&](context_t& context) {
     detail::sorted_search_launch<bounds_lower, search_launch_t>(a, a_count,
-      b, b_count, ws.lower, less_t<int>(), ws.partitions, context);
+      b, b_count, ws.lower, less_t<int>(), ws.partitions, ws.samples,
+      context);
     detail::sorted_search_launch<bounds_upper, search_launch_t>(a, a_count,
-      b, b_count, ws.upper, less_t<int>(), ws.partitions, context);
+      b, b_count, ws.upper, less_t<int>(), ws.partitions, ws.samples,
+      context);
     detail::scan_launch<scan_type_exc, scan_launch_t>(
       make_load_iterator<int>(match_count_f { ws.lower, ws.upper }), a_count,
       ws.starts, plus_t<int>(), join_count, ws.partials, context);

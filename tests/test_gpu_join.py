@@ -53,3 +53,46 @@ def test_inner_join_matches_oracle(oracle, dev, na, nb, hi):
     want = oracle.inner_join(a, b)
     assert tuple(got.shape) == want.shape
     assert np.array_equal(got.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("n,h,hi", [
+    (3 * (1 << 20) + 5, (1 << 21) + 3, 1 << 24),      # few ties
+    ((1 << 22) + 1, 1023, 1 << 20),                   # a haystack shorter than one sample step
+    (1025, (1 << 22) + 77, 1 << 20),                  # ... and needles
+    ((1 << 21) + 1000, (1 << 21) + 24, 7),            # runs of equal keys far longer than a tile
+    (5 << 20, 3 << 20, 1 << 30)])
+def test_sorted_search_large_inputs_take_the_sampled_partition(dev, n, h, hi):
+    """From 2^22 keys on the tile splits are searched over every 1,024th key
+    first (and then inside one window of the inputs); results against numpy."""
+    import moderngpu_amd as m
+    rng = np.random.default_rng(n + 3 * h)
+    needles, haystack = _keys(rng, n, hi), _keys(rng, h, hi)
+    d_needles, d_haystack = torch.from_numpy(needles).to(dev), torch.from_numpy(haystack).to(dev)
+    for bounds, side in (("lower", "left"), ("upper", "right")):
+        got = m.sorted_search(d_needles, d_haystack, bounds)
+        torch.cuda.synchronize()
+        assert np.array_equal(got.cpu().numpy(), np.searchsorted(haystack, needles, side=side)), bounds
+
+
+def test_sorted_search_large_disjoint_and_interleaved(dev):
+    import moderngpu_amd as m
+    n = (3 << 20) + 11
+    low = np.arange(n, dtype=np.int32)
+    high = np.arange(n, dtype=np.int32) + (1 << 28)
+    even, odd = 2 * np.arange(n, dtype=np.int32), 2 * np.arange(n, dtype=np.int32) + 1
+    for needles, haystack in ((low, high), (high, low), (even, odd), (odd, even), (even, even)):
+        for bounds, side in (("lower", "left"), ("upper", "right")):
+            got = m.sorted_search(torch.from_numpy(needles).to(dev),
+                                  torch.from_numpy(haystack).to(dev), bounds)
+            assert np.array_equal(got.cpu().numpy(),
+                                  np.searchsorted(haystack, needles, side=side))
+
+
+def test_inner_join_large(oracle, dev):
+    import moderngpu_amd as m
+    rng = np.random.default_rng(77)
+    a, b = _keys(rng, (1 << 22) + 9, 1 << 22), _keys(rng, (1 << 21) + 1, 1 << 22)
+    got = m.inner_join(torch.from_numpy(a).to(dev), torch.from_numpy(b).to(dev))
+    want = oracle.inner_join(a, b)
+    assert tuple(got.shape) == want.shape
+    assert np.array_equal(got.cpu().numpy(), want)
