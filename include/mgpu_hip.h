@@ -281,7 +281,8 @@ MGPU_HIP_API int mgpu_hip_workcreate_downsweep(const int* created, int count,
 
 /* ---- sorted search and join (callers of the search) ---------------------- */
 
-/* Bytes of workspace mgpu_hip_sorted_search needs (the tile splits). */
+/* Bytes of workspace mgpu_hip_sorted_search needs (the tile splits and, for
+ * inputs of 2^22 keys or more, every 1,024th key of both inputs). */
 MGPU_HIP_API size_t mgpu_hip_sorted_search_workspace_bytes(int num_needles,
   int num_haystack);
 
