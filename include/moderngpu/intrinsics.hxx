@@ -158,6 +158,15 @@ MGPU_DEVICE inline type_t readlane(type_t x, int lane) {
   return s.get();
 }
 
+// Pins the point at which x has to be in registers: the compiler may not
+// move the load that produces x below this call (it otherwise sinks a load
+// into the branch that uses it, behind the wait for everything else).
+template<typename type_t>
+MGPU_DEVICE inline void needed_here(const type_t& x) {
+  lane_words_t<type_t> s(x);
+  asm volatile("" :: "v"(s.w[0]));
+}
+
 template<typename type_t>
 MGPU_DEVICE inline type_t bpermute(type_t x, int src_lane) {
   lane_words_t<type_t> s(x);

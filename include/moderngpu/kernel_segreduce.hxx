@@ -523,10 +523,12 @@ struct segreduce_spine_f {
 
   MGPU_DEVICE void operator()(int tid, int cta) const {
     typedef cta_segscan_t<nt, type_t> segscan_t;
-    typedef cta_reduce_t<nt, type_t> reduce_t;
     __shared__ union {
       typename segscan_t::storage_t segscan;
-      typename reduce_t::storage_t reduce;
+      struct {
+        type_t totals[nt / warp_size];
+        bool have[nt / warp_size];
+      } fold;
     } shared;
     __shared__ int open_first;
 
@@ -563,27 +565,77 @@ struct segreduce_spine_f {
 
     int first = open_first;
     if(first >= 0 && first < base) {
-      // Ordered fold of carries [first, base): a contiguous chunk per thread.
+      // Ordered fold of carries [first, base).  A lane takes vt consecutive
+      // carries (32 bytes), a wavefront row 64 such chunks; a row is read
+      // with full-width loads, folded per lane and then across the lanes in
+      // order.  A wavefront takes a contiguous block of rows, a batch of
+      // them in flight at a time, and folds their totals in order; thread 0
+      // folds the wavefronts' results in order.
+      enum {
+        num_waves = nt / warp_size,
+        vt = sizeof(type_t) <= 16 ? 32 / sizeof(type_t) : 1,
+        batch = sizeof(type_t) <= 32 ? 8 : 4
+      };
+      int lane = tid % warp_size, wave = tid / warp_size;
       int len = base - first;
-      int chunk = div_up(len, nt);
-      int active = div_up(len, chunk);
-      int at = first + chunk * tid;
+      int chunks = div_up(len, (int)vt);
+      int rows = div_up(chunks, (int)warp_size);
+      int rows_per_wave = div_up(rows, (int)num_waves);
+      int row0 = rows_per_wave * wave;
+      int row1 = min(row0 + rows_per_wave, rows);
       type_t x = init;
-      if(tid < active) {
-        // Blocks of eight independent loads, folded in order.
-        x = values[at];
-        for(int k0 = 1; k0 < chunk; k0 += 8) {
-          type_t y[8];
+      bool have = false;
+      for(int r0 = row0; r0 < row1; r0 += batch) {
+        // Every load is issued before the first row is folded.  A chunk past
+        // the end repeats the last one; the last chunk is moved back to end
+        // at `base` (base >= nt > vt, so it stays inside the array) and the
+        // skip carries in front of its own part are left out of the fold.
+        type_t y[batch][vt];
+        int skip[batch];
+        PRAGMA_UNROLL
+        for(int k = 0; k < batch; ++k) {
+          int at = vt * min(warp_size * (r0 + k) + lane, chunks - 1);
+          int from = min(at, len - vt);
+          skip[k] = at - from;
           PRAGMA_UNROLL
-          for(int k = 0; k < 8; ++k)
-            if(k0 + k < chunk && at + k0 + k < base) y[k] = values[at + k0 + k];
+          for(int j = 0; j < vt; ++j)
+            y[k][j] = values[first + from + j];
+        }
+        PRAGMA_UNROLL
+        for(int k = 0; k < batch; ++k)
+          detail::needed_here(y[k][0]);
+        PRAGMA_UNROLL
+        for(int k = 0; k < batch; ++k) {
+          type_t folded = y[k][0];
           PRAGMA_UNROLL
-          for(int k = 0; k < 8; ++k)
-            if(k0 + k < chunk && at + k0 + k < base) x = op(x, y[k]);
+          for(int j = 1; j < vt; ++j)
+            folded = (j <= skip[k]) ? y[k][j] : op(folded, y[k][j]);
+          int valid = min(chunks - warp_size * (r0 + k), (int)warp_size);
+          type_t total = detail::readlane(wave_scan(folded, op, lane),
+            max(valid, 1) - 1);
+          if(r0 + k < row1) {
+            x = have ? op(x, total) : total;
+            have = true;
+          }
         }
       }
-      type_t front = reduce_t().reduce(tid, x, shared.reduce, active, op, true);
-      if(open_run) value = op(front, value);
+      if(!lane) {
+        shared.fold.totals[wave] = x;
+        shared.fold.have[wave] = have;
+      }
+      __syncthreads();
+      if(open_run) {
+        type_t front = init;
+        bool any = false;
+        PRAGMA_UNROLL
+        for(int w = 0; w < num_waves; ++w)
+          if(shared.fold.have[w]) {
+            front = any ? op(front, shared.fold.totals[w]) :
+              shared.fold.totals[w];
+            any = true;
+          }
+        value = op(front, value);
+      }
     }
 
     if(run_end) output[seg] = combine ? op(old, value) : value;
