@@ -130,7 +130,8 @@ MGPU_HIP_API int mgpu_hip_segreduce_static(const void* input, int count,
 
 /* Same, running only the selected phases (MGPU_PHASE_*).  A later phase uses
  * what an earlier complete call left in the same workspace.  For timing the
- * partition, tile and spine kernels separately. */
+ * partition, tile and spine kernels separately.  (Inputs of up to 4,096
+ * tiles have no partition kernel: their tile kernel finds its own splits.) */
 MGPU_HIP_API int mgpu_hip_segreduce_phases(const void* input, int count,
   const int* segments, int num_segments, void* output, int dtype, int op,
   const void* init, void* workspace, size_t workspace_bytes,
