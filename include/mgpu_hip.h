@@ -180,6 +180,9 @@ MGPU_HIP_API size_t mgpu_hip_lbs_workspace_bytes(int count, int num_segments);
 MGPU_HIP_API int mgpu_hip_load_balance_search(int count, const int* segments,
   int num_segments, int* output, void* workspace, size_t workspace_bytes,
   mgpu_stream_t stream);
+/* Same with the phases selected (MGPU_PHASE_PARTITION, MGPU_PHASE_TILES).
+ * Calls of up to 1,536 tiles have no partition kernel: their tile kernel
+ * finds its own splits. */
 MGPU_HIP_API int mgpu_hip_load_balance_search_phases(int count,
   const int* segments, int num_segments, int* output, void* workspace,
   size_t workspace_bytes, mgpu_stream_t stream, int phases);

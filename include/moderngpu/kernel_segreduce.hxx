@@ -247,8 +247,13 @@ struct tile_source_storage_t<lbs_input_t<func_t, pointers_t, type_t>, nt,
 ////////////////////////////////////////////////////////////////////////////////
 // K2
 
+// own_splits: launched without a partition array, the tile finds its two
+// splits itself (calls of few tiles, see segreduce_launch).  A separate
+// instantiation, because the search in front costs the kernel of large
+// calls time even when it is only branched around (2^26 floats: 49.8
+// against 49.2 us per call).
 template<typename launch_t, typename input_it, typename segments_it,
-  typename output_it, typename op_t, typename type_t>
+  typename output_it, typename op_t, typename type_t, bool own_splits = false>
 struct segreduce_tile_f {
   input_it input;
   int count;
@@ -295,24 +300,24 @@ struct segreduce_tile_f {
     __shared__ storage_t shared;
 
     int mp0, mp1;
-    if(mp_data) {
+    if constexpr(!own_splits) {
       mp0 = mp_data[cta];
       mp1 = mp_data[cta + 1];
     } else {
       // No partition kernel has run: one wavefront per end of the tile
-      // finds the split itself.
-      __shared__ int own_splits[2];
+      // finds the split.
+      __shared__ int own[2];
       int total = count + num_segments;
       for(int end = tid / warp_size; end < 2; end += nt / warp_size) {
         int diag = (int)min((int64_t)nv * (cta + end), (int64_t)total);
         int split = merge_path_wave<bounds_upper>(
           counting_iterator_t<int>(0), count, segments, num_segments, diag,
           less_t<int>(), tid % warp_size);
-        if(0 == tid % warp_size) own_splits[end] = split;
+        if(0 == tid % warp_size) own[end] = split;
       }
       __syncthreads();
-      mp0 = own_splits[0];
-      mp1 = own_splits[1];
+      mp0 = own[0];
+      mp1 = own[1];
     }
     merge_range_t range = tile_range(count, num_segments, cta, nv, mp0, mp1);
     // A tile that lies nv items or more in front of the end of the input
@@ -716,14 +721,19 @@ void segreduce_launch(input_it input, int count, segments_it segments,
   // 2^26 floats in segments of 64: 6.5 against 10.0 us up to 2^18, 19.4
   // against 20.4 us at 2^24 (4,160 tiles), 32.9 against 30.1 us at 2^25.
   enum { own_splits_max_tiles = 4096 };
-  if(ws.num_ctas <= own_splits_max_tiles) mp_data = nullptr;
-  else if(phases & phase_partition)
+  bool own_splits = ws.num_ctas <= own_splits_max_tiles;
+  if(!own_splits && (phases & phase_partition))
     load_balance_partitions_into((int64_t)count, segments, num_segments,
       cta_dim.nv(), mp_data, context);
 
   type_t* carry_values = (type_t*)(base + ws.values_offset);
   int* carry_codes = (int*)(base + ws.codes_offset);
-  if(phases & phase_tiles) {
+  if((phases & phase_tiles) && own_splits) {
+    segreduce_tile_f<launch_t, input_it, segments_it, output_it, op_t, type_t,
+      true> k_reduce { input, count, segments, num_segments, output, op,
+        init, nullptr, carry_values, carry_codes, ws.num_ctas };
+    cta_launch<launch_t>(k_reduce, xcd_grid(ws.num_ctas), context, args...);
+  } else if(phases & phase_tiles) {
     segreduce_tile_f<launch_t, input_it, segments_it, output_it, op_t, type_t>
       k_reduce { input, count, segments, num_segments, output, op, init,
         mp_data, carry_values, carry_codes, ws.num_ctas };

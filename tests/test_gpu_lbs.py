@@ -103,6 +103,26 @@ def test_lbs_layouts(dev, oracle):
         assert np.array_equal(rank.cpu().numpy(), wrank), name
 
 
+@pytest.mark.parametrize("tiles", [1536, 1537])
+def test_either_side_of_the_partition_kernel(dev, oracle, tiles):
+    """Calls of up to 1,536 tiles let the tile kernel find its own splits;
+    one tile more and a partition kernel runs first."""
+    import moderngpu_amd as m
+    rng = np.random.default_rng(32)
+    for spacing, expand in ((m.lbs_search_tile_size(), False), (m.lbs_tile_size(), True)):
+        nseg = 700_000
+        count = (tiles - 1) * spacing + 1 - nseg
+        assert (count + nseg + spacing - 1) // spacing == tiles
+        segs = random_segments(rng, count, nseg)
+        if expand:
+            vals = rng.integers(0, 2 ** 31, size=nseg).astype(np.int32)
+            got = m.interval_expand(_dev(vals), count, _dev(segs)).cpu().numpy()
+            assert np.array_equal(got, oracle.interval_expand(vals, count, segs))
+        else:
+            got = m.load_balance_search(count, _dev(segs)).cpu().numpy()
+            assert np.array_equal(got, oracle.load_balance_search(count, segs))
+
+
 @pytest.mark.parametrize("elem", [np.uint8, np.int16, np.int32, np.float64, "b16"])
 def test_interval_expand(dev, oracle, elem):
     import torch

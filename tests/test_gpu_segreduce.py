@@ -167,6 +167,22 @@ def test_spine_levels(dev, oracle):
         _check(values, np.array(segs, dtype=np.int32), "maximum", -3, oracle, str(segs))
 
 
+@pytest.mark.parametrize("tiles", [4096, 4097])
+def test_either_side_of_the_partition_kernel(dev, oracle, tiles):
+    """Calls of up to 4,096 tiles let every tile find its own splits; one tile
+    more and the partition kernel runs.  Same input but for one value."""
+    import moderngpu_amd as m
+    rng = np.random.default_rng(31)
+    nv = m.segreduce_tile_size(0)
+    nseg = 300_000
+    count = tiles * nv - nseg - nv + 1          # count + nseg = (tiles - 1) * nv + 1
+    assert (count + nseg + nv - 1) // nv == tiles
+    segs = random_segments(rng, count, nseg)
+    values = rng.integers(-1000, 1000, size=count).astype(np.int32)
+    _check(values, segs, "plus", 7, oracle, "tiles=%d" % tiles)
+    _check(values.astype(np.float32), segs, "maximum", -1.0, oracle, "tiles=%d" % tiles)
+
+
 def test_full_size_config2_properties(dev):
     """2^26 fp32 items: compared on the device with torch.segment_reduce
     (independent code) in float64, tolerance 1e-5 * sum|x|."""
