@@ -302,7 +302,8 @@ MGPU_HIP_API int mgpu_hip_sorted_search(const int* needles, int num_needles,
  * steps its data-dependent output size forces (the reference reads the count
  * back and allocates in between, :33-36).
  *
- * Step 1 (sorted searches + scan of the match counts, :14-31): stores the
+ * Step 1 (one sorted search for lower bounds and match counts where the
+ * reference runs two searches, and the scan of the counts, :14-31): stores the
  * number of pairs to *join_count (device memory, or host memory the device
  * can write) and leaves what step 2 needs in `workspace`
  * (mgpu_hip_inner_join_workspace_bytes(a_count, b_count) bytes). */

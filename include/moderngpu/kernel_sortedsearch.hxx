@@ -26,10 +26,19 @@ namespace detail {
 typedef launch_box_t<arch_gfx950_cta<256, 12, 12> >
   sorted_search_launch_default_t;
 
+// with_counts (bounds_lower only): the kernel also writes, for every needle,
+// how many haystack keys are equivalent to it -- upper bound minus lower
+// bound, what a join needs -- from a second search over the same LDS keys.
+// The run of equivalent keys may go on behind the tile's haystack range, so
+// up to `beyond` further keys are staged with it; a needle whose run
+// outlasts those too finishes its search in global memory.
 template<bounds_t bounds, typename launch_t, typename needles_it,
-  typename haystack_it, typename indices_it, typename comp_t>
+  typename haystack_it, typename indices_it, typename comp_t,
+  bool with_counts = false>
 struct sorted_search_f {
   typedef typename std::iterator_traits<needles_it>::value_type type_t;
+  static_assert(!with_counts || bounds_lower == bounds,
+    "match counts go with lower bounds");
   needles_it needles;
   int num_needles;
   haystack_it haystack;
@@ -38,15 +47,20 @@ struct sorted_search_f {
   comp_t comp;
   const int* mp_data;
   int num_tiles;
+  int* counts;
 
   MGPU_DEVICE void operator()(int tid, int cta) const {
     typedef typename launch_t::sm_ptx params_t;
     enum {
       nt = params_t::nt, vt = params_t::vt, nv = nt * vt,
-      // LDS keys: the first power of two that holds a tile.
-      padded = (nv & (nv - 1)) ? (2 << s_log2((int)nv)) : nv,
+      beyond = with_counts ? 64 : 0,
+      // LDS keys: the first power of two that holds a tile (and the keys
+      // staged behind it).
+      room = nv + beyond,
+      padded = (room & (room - 1)) ? (2 << s_log2((int)room)) : room,
       lanes = 2                     // searches a thread runs side by side
     };
+    static_assert(beyond <= nt, "one more key per thread at most");
     int tile = xcd_tile(cta, num_tiles);
     if(tile >= num_tiles) return;
     __shared__ type_t keys[padded];
@@ -59,22 +73,28 @@ struct sorted_search_f {
     if(!a_count) return;            // b_count <= nv - 1 from here on
 
     // All global loads of the thread are issued before the first of them is
-    // used.  Behind the tile's haystack keys the LDS array repeats the last
+    // used.  Behind the staged haystack keys the LDS array repeats the last
     // of them up to its padded size: a probe past the end then answers like
     // the last key, the search needs no bounds test, and what it finds is
     // clipped to b_count afterwards.
-    type_t hay[vt], needle[vt];
+    // staged = haystack keys in LDS: the tile's own and up to `beyond` more.
+    int staged = min(b_count + (int)beyond, num_haystack - range.b_begin);
+    type_t hay[vt], needle[vt], hay_beyond;
     PRAGMA_UNROLL
     for(int i = 0; i < vt; ++i)
       if(nt * i + tid < b_count)
         hay[i] = haystack[range.b_begin + nt * i + tid];
+    if(with_counts && b_count + tid < staged)
+      hay_beyond = haystack[range.b_begin + b_count + tid];
     PRAGMA_UNROLL
     for(int i = 0; i < vt; ++i)
       if(nt * i + tid < a_count)
         needle[i] = needles[range.a_begin + nt * i + tid];
-    if(b_count) {
-      type_t filler = haystack[range.b_begin + b_count - 1];
-      for(int j = b_count + tid; j < padded; j += nt) keys[j] = filler;
+    if(staged) {
+      type_t filler = haystack[range.b_begin + staged - 1];
+      if(with_counts && b_count + tid < staged)
+        keys[b_count + tid] = hay_beyond;
+      for(int j = staged + tid; j < padded; j += nt) keys[j] = filler;
     }
     PRAGMA_UNROLL
     for(int i = 0; i < vt; ++i)
@@ -107,12 +127,48 @@ struct sorted_search_f {
           if(in_front) at[l] += step * sizeof(type_t);
         }
       }
+      // The same over "keys not behind the needle": the upper bound.
+      unsigned up[lanes];
+      if constexpr(with_counts) {
+        PRAGMA_UNROLL
+        for(int l = 0; l < lanes; ++l) up[l] = 0;
+        PRAGMA_UNROLL
+        for(int step = padded / 2; step >= 1; step >>= 1) {
+          type_t key[lanes];
+          PRAGMA_UNROLL
+          for(int l = 0; l < lanes; ++l)
+            key[l] = *(const type_t*)((const char*)keys + up[l] +
+              (step - 1) * sizeof(type_t));
+          PRAGMA_UNROLL
+          for(int l = 0; l < lanes; ++l) {
+            const type_t& mine = needle[i0 + l < vt ? i0 + l : vt - 1];
+            if(!comp(mine, key[l])) up[l] += step * sizeof(type_t);
+          }
+        }
+      }
       PRAGMA_UNROLL
       for(int l = 0; l < lanes; ++l) {
         int p = nt * (i0 + l) + tid;
-        if(i0 + l < vt && p < a_count)
-          indices[range.a_begin + p] = range.b_begin +
-            min((int)(at[l] / sizeof(type_t)), b_count);
+        if(i0 + l < vt && p < a_count) {
+          int lower = min((int)(at[l] / sizeof(type_t)), b_count);
+          indices[range.a_begin + p] = range.b_begin + lower;
+          if constexpr(with_counts) {
+            int upper = range.b_begin + (int)(up[l] / sizeof(type_t));
+            if(upper >= range.b_begin + staged) {
+              // Every staged key is equivalent to the needle or in front of
+              // it: the run ends somewhere behind them.
+              const type_t& mine = needle[i0 + l < vt ? i0 + l : vt - 1];
+              int lo = range.b_begin + staged, hi = num_haystack;
+              while(lo < hi) {
+                int mid = (int)(((unsigned)lo + (unsigned)hi) / 2);
+                if(!comp(mine, haystack[mid])) lo = mid + 1;
+                else hi = mid;
+              }
+              upper = lo;
+            }
+            counts[range.a_begin + p] = upper - (range.b_begin + lower);
+          }
+        }
       }
     }
   }
@@ -207,13 +263,15 @@ struct sampled_partition_f {
 // Splits in caller-provided device memory: div_up(num_needles +
 // num_haystack, nv) + 1 ints, and sorted_search_sample_count() keys (or
 // null: the splits are then found by plain binary searches).
+// counts: null, or (bounds_lower) where the number of haystack keys
+// equivalent to each needle goes.
 template<bounds_t bounds, typename launch_t, typename needles_it,
   typename haystack_it, typename indices_it, typename comp_t>
 void sorted_search_launch(needles_it needles, int num_needles,
   haystack_it haystack, int num_haystack, indices_it indices, comp_t comp,
   int* mp_data,
   typename std::iterator_traits<needles_it>::value_type* samples,
-  context_t& context) {
+  context_t& context, int* counts = nullptr) {
   typedef typename std::iterator_traits<needles_it>::value_type type_t;
   int64_t total = (int64_t)num_needles + num_haystack;
   if(total >= ((int64_t)1 << 31)) throw cuda_exception_t(hipErrorInvalidValue);
@@ -234,9 +292,18 @@ void sorted_search_launch(needles_it needles, int num_needles,
   } else
     merge_path_partitions_into<bounds>(needles, (int64_t)num_needles,
       haystack, (int64_t)num_haystack, (int64_t)nv, comp, mp_data, context);
+  if constexpr(bounds_lower == bounds) {
+    if(counts) {
+      sorted_search_f<bounds, launch_t, needles_it, haystack_it, indices_it,
+        comp_t, true> k { needles, num_needles, haystack, num_haystack,
+          indices, comp, mp_data, num_tiles, counts };
+      cta_launch<launch_t>(k, xcd_grid(num_tiles), context);
+      return;
+    }
+  }
   sorted_search_f<bounds, launch_t, needles_it, haystack_it, indices_it,
     comp_t> k { needles, num_needles, haystack, num_haystack, indices, comp,
-      mp_data, num_tiles };
+      mp_data, num_tiles, nullptr };
   cta_launch<launch_t>(k, xcd_grid(num_tiles), context);
 }
 

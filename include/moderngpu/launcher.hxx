@@ -296,6 +296,34 @@ bool launcher_sorted_search(bool upper, needles_it needles, int num_needles,
     return false;
 }
 
+// inner_join of int keys ordered by less_t<int>: both steps of the layer,
+// with the count read back in between as the header-only path does.
+template<typename launch_arg_t, typename a_it, typename b_it, typename comp_t>
+bool launcher_inner_join(a_it a, int a_count, b_it b, int b_count, comp_t,
+  context_t& context, mem_t<int2>& output) {
+  if constexpr(std::is_same<launch_arg_t, empty_t>::value &&
+    std::is_same<comp_t, less_t<int> >::value &&
+    launcher_points_to_t<a_it, int>::value &&
+    launcher_points_to_t<b_it, int>::value) {
+    size_t bytes = mgpu_hip_inner_join_workspace_bytes(a_count, b_count);
+    mem_t<char> workspace(bytes, context);
+    mem_t<int> total(1, context);
+    launcher_check(mgpu_hip_inner_join_count(a, a_count, b, b_count,
+      total.data(), workspace.data(), bytes, context.stream()));
+    int join_count = from_mem(total)[0];
+    output = mem_t<int2>(join_count, context);
+    size_t pairs_bytes = mgpu_hip_inner_join_pairs_workspace_bytes(a_count,
+      join_count);
+    mem_t<char> pairs_workspace(pairs_bytes, context);
+    launcher_check(mgpu_hip_inner_join_pairs(a_count, b_count, join_count,
+      workspace.data(), (int*)output.data(), pairs_workspace.data(),
+      pairs_bytes, context.stream()));
+    ++launcher_calls();
+    return true;
+  } else
+    return false;
+}
+
 // load_balance_partitions into an int array.
 template<typename segments_it>
 bool launcher_load_balance_partitions(int64_t count, segments_it segments,
@@ -327,6 +355,8 @@ template<typename launch_arg_t, typename... args_t>
 constexpr bool launcher_reduce(const args_t&...) { return false; }
 template<typename launch_arg_t, typename... args_t>
 constexpr bool launcher_sorted_search(const args_t&...) { return false; }
+template<typename launch_arg_t, typename... args_t>
+constexpr bool launcher_inner_join(const args_t&...) { return false; }
 template<typename... args_t>
 constexpr bool launcher_load_balance_partitions(const args_t&...) {
   return false;

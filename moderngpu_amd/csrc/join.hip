@@ -31,7 +31,7 @@ size_t search_samples_offset(int num_needles, int num_haystack) {
 // Temporaries of mgpu_hip_inner_join_count, which mgpu_hip_inner_join_pairs
 // reads again.
 struct join_workspace_t {
-  int* lower; int* upper; int* starts; int* partitions; int* samples;
+  int* lower; int* matches; int* starts; int* partitions; int* samples;
   int* partials;
   size_t bytes;
   join_workspace_t(int a_count, int b_count, void* base) {
@@ -42,7 +42,7 @@ struct join_workspace_t {
       return p;
     };
     lower = take(a_count);
-    upper = take(a_count);
+    matches = take(a_count);
     starts = take(a_count);
     partitions = take(search_partitions(a_count, b_count));
     samples = take(search_samples(a_count, b_count));
@@ -50,11 +50,6 @@ struct join_workspace_t {
       scan_launch_t::sm_ptx::nt * scan_launch_t::sm_ptx::vt));
     bytes = (size_t)(at - (char*)base);
   }
-};
-
-struct match_count_f {
-  const int* lower; const int* upper;
-  MGPU_DEVICE int operator()(int i) const { return upper[i] - lower[i]; }
 };
 
 bool keys_ok(const int* a, int a_count, const int* b, int b_count) {
@@ -111,15 +106,15 @@ int mgpu_hip_inner_join_count(const int* a, int a_count, const int* b,
   if(ws.bytes && (!workspace || workspace_bytes < ws.bytes))
     return (int)hipErrorInvalidValue;
   return guarded(stream, [&](context_t& context) {
-    detail::sorted_search_launch<bounds_lower, search_launch_t>(a, a_count,
-      b, b_count, ws.lower, less_t<int>(), ws.partitions, ws.samples,
-      context);
-    detail::sorted_search_launch<bounds_upper, search_launch_t>(a, a_count,
-      b, b_count, ws.upper, less_t<int>(), ws.partitions, ws.samples,
-      context);
+    // One search: the lower bound of every a key and the number of b keys
+    // equal to it.
+    if(a_count)
+      detail::sorted_search_launch<bounds_lower, search_launch_t>(a, a_count,
+        b, b_count, ws.lower, less_t<int>(), ws.partitions, ws.samples,
+        context, ws.matches);
     detail::scan_launch<scan_type_exc, scan_launch_t>(
-      make_load_iterator<int>(match_count_f { ws.lower, ws.upper }), a_count,
-      ws.starts, plus_t<int>(), join_count, ws.partials, context);
+      (const int*)ws.matches, a_count, ws.starts, plus_t<int>(), join_count,
+      ws.partials, context);
   });
 }
 

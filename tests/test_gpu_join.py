@@ -43,7 +43,10 @@ def test_sorted_search_disjoint_ranges(oracle, dev):
 
 @pytest.mark.parametrize("na,nb,hi", [
     (0, 0, 3), (0, 50, 3), (50, 0, 3), (1000, 1000, 10000), (5000, 4000, 100),
-    (300, 200, 0), (200000, 150000, 1 << 16), (1 << 20, 1 << 20, 1 << 20)])
+    (300, 200, 0), (200000, 150000, 1 << 16), (1 << 20, 1 << 20, 1 << 20),
+    # runs of equal b keys that go on far behind the tile in which they begin:
+    # the match count of an a key is finished outside the tile's own keys
+    (3000, 6000, 3), (20000, 20000, 50), (40, 100000, 1)])
 def test_inner_join_matches_oracle(oracle, dev, na, nb, hi):
     import moderngpu_amd as m
     rng = np.random.default_rng(na * 17 + nb)
