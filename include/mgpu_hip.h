@@ -47,7 +47,10 @@ enum { MGPU_PLUS = 0, MGPU_MAXIMUM = 1, MGPU_MINIMUM = 2 };
 enum { MGPU_BOUNDS_LOWER = 0, MGPU_BOUNDS_UPPER = 1 };
 /* Phase masks for the *_phases entry points (measurement only). */
 enum { MGPU_PHASE_PARTITION = 1, MGPU_PHASE_TILES = 2, MGPU_PHASE_SPINE = 4,
-       MGPU_PHASE_ALL = 7 };
+       MGPU_PHASE_ALL = 7,
+       /* or-ed in: run the partition kernel also for calls small enough to
+        * do without it (see the *_phases functions) */
+       MGPU_PHASE_PARTITION_ALWAYS = 8 };
 
 /* Library version, major * 10000 + minor * 100 + patch. */
 MGPU_HIP_API int mgpu_hip_version(void);
@@ -131,7 +134,8 @@ MGPU_HIP_API int mgpu_hip_segreduce_static(const void* input, int count,
 /* Same, running only the selected phases (MGPU_PHASE_*).  A later phase uses
  * what an earlier complete call left in the same workspace.  For timing the
  * partition, tile and spine kernels separately.  (Inputs of up to 4,096
- * tiles have no partition kernel: their tile kernel finds its own splits.) */
+ * tiles have no partition kernel: their tile kernel finds its own splits,
+ * unless MGPU_PHASE_PARTITION_ALWAYS is or-ed into phases.) */
 MGPU_HIP_API int mgpu_hip_segreduce_phases(const void* input, int count,
   const int* segments, int num_segments, void* output, int dtype, int op,
   const void* init, void* workspace, size_t workspace_bytes,
@@ -182,7 +186,7 @@ MGPU_HIP_API int mgpu_hip_load_balance_search(int count, const int* segments,
   mgpu_stream_t stream);
 /* Same with the phases selected (MGPU_PHASE_PARTITION, MGPU_PHASE_TILES).
  * Calls of up to 1,536 tiles have no partition kernel: their tile kernel
- * finds its own splits. */
+ * finds its own splits, unless MGPU_PHASE_PARTITION_ALWAYS is or-ed in. */
 MGPU_HIP_API int mgpu_hip_load_balance_search_phases(int count,
   const int* segments, int num_segments, int* output, void* workspace,
   size_t workspace_bytes, mgpu_stream_t stream, int phases);

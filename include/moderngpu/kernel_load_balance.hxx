@@ -381,7 +381,11 @@ inline int lbs_total(int count, int num_segments) {
   return (int)total;
 }
 
-enum { lbs_phase_partition = 1, lbs_phase_tiles = 2, lbs_phase_all = 3 };
+enum {
+  lbs_phase_partition = 1, lbs_phase_tiles = 2, lbs_phase_all = 3,
+  // The partition kernel runs whatever the size of the call.
+  lbs_phase_partition_always = 8
+};
 
 // Ints of partition storage for `total` merged elements cut into tiles of nv:
 // one (items, starts) pair per split.
@@ -421,7 +425,8 @@ void transform_lbs_launch(func_t f, int count, segments_it segments,
   int num_tiles = div_up(total, lbs_tile_spacing(nv));
 
   enum { own_splits_max_tiles = 1536 };
-  if(num_tiles <= own_splits_max_tiles) {
+  if(num_tiles <= own_splits_max_tiles &&
+    !(phases & lbs_phase_partition_always)) {
     // A call of few tiles is bound by its launches: the tile kernel finds
     // its own splits and no partition kernel runs.  load_balance_search over
     // segments of 16 items: 5.6 against 7.4 us for 2^14 items, 7.0 against

@@ -696,7 +696,10 @@ enum {
   phase_partition = 1,    // K1
   phase_tiles = 2,        // K2
   phase_spine = 4,        // K3
-  phase_all = 7
+  phase_all = 7,
+  // With this bit the partition kernel runs whatever the size of the call
+  // (tests and measurements of that path on small inputs).
+  phase_partition_always = 8
 };
 
 // Launches K1, K2 and the spine into caller-provided workspace.  `phases`
@@ -721,7 +724,8 @@ void segreduce_launch(input_it input, int count, segments_it segments,
   // 2^26 floats in segments of 64: 6.5 against 10.0 us up to 2^18, 19.4
   // against 20.4 us at 2^24 (4,160 tiles), 32.9 against 30.1 us at 2^25.
   enum { own_splits_max_tiles = 4096 };
-  bool own_splits = ws.num_ctas <= own_splits_max_tiles;
+  bool own_splits = ws.num_ctas <= own_splits_max_tiles &&
+    !(phases & phase_partition_always);
   if(!own_splits && (phases & phase_partition))
     load_balance_partitions_into((int64_t)count, segments, num_segments,
       cta_dim.nv(), mp_data, context);

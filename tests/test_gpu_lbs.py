@@ -94,9 +94,11 @@ def test_lbs_layouts(dev, oracle):
     layouts = list(segment_layouts(rng, m.lbs_search_tile_size())) + \
         list(segment_layouts(rng, m.lbs_tile_size()))
     for name, count, segs in layouts:
-        got = m.load_balance_search(count, _dev(segs)).cpu().numpy()
         want = oracle.load_balance_search(count, segs)
-        assert np.array_equal(got, want), name
+        # small calls find their own splits; 3 | 8 puts the partition kernel in front
+        for phases in (3, 3 | 8):
+            got = m.load_balance_search(count, _dev(segs), phases=phases).cpu().numpy()
+            assert np.array_equal(got, want), (name, phases)
         seg, rank = m.transform_lbs(count, _dev(segs))
         wseg, wrank = oracle.transform_lbs(count, segs)
         assert np.array_equal(seg.cpu().numpy(), wseg), name
@@ -140,6 +142,8 @@ def test_interval_expand(dev, oracle, elem):
             vals = rng.integers(0, 120, size=nseg).astype(elem)
             got = m.interval_expand(_dev(vals), count, _dev(segs)).cpu().numpy()
             want = oracle.interval_expand(vals, count, segs)
+            parted = m.interval_expand(_dev(vals), count, _dev(segs), phases=3 | 8)
+            assert np.array_equal(parted.cpu().numpy(), want), name + "/partitioned"
         assert np.array_equal(got, want), name
 
 

@@ -23,7 +23,7 @@ def _dev(a):
     return torch.from_numpy(np.ascontiguousarray(a)).cuda()
 
 
-def _gpu_segreduce(values, segs, op, init):
+def _gpu_segreduce(values, segs, op, init, phases=7):
     import torch
     import moderngpu_amd as m
     unsigned = values.dtype in (np.uint32, np.uint64)
@@ -31,7 +31,7 @@ def _gpu_segreduce(values, segs, op, init):
     # Poison the output so segments nobody writes are noticed.
     out = torch.full((segs.size,), 0x5a5a5a5a if v.dtype.kind in "iu" else float("nan"),
                      dtype=_dev(v[:0]).dtype, device="cuda")
-    m.segreduce(_dev(v), _dev(segs), op, init, out=out, unsigned=unsigned)
+    m.segreduce(_dev(v), _dev(segs), op, init, out=out, unsigned=unsigned, phases=phases)
     got = out.cpu().numpy()
     return got.view(values.dtype) if unsigned else got
 
@@ -45,8 +45,8 @@ def _abs_sums(values, segs):
     return out
 
 
-def _check(values, segs, op, init, oracle, name=""):
-    got = _gpu_segreduce(values, segs, op, init)
+def _check(values, segs, op, init, oracle, name="", phases=7):
+    got = _gpu_segreduce(values, segs, op, init, phases)
     want = oracle.segreduce(values, segs, op, init)
     if values.dtype.kind == "f" and op == "plus":
         # "exact": extended-precision (x87 long double) sum of the same inputs.
@@ -114,7 +114,10 @@ def test_layouts_all_types(dev, oracle, dtype, op):
             info = np.iinfo(dtype)
             values = rng.integers(info.min, info.max, size=count, dtype=dtype, endpoint=True)
             init = 42
+        # as the call runs (small calls: tiles that find their own splits),
+        # and with the partition kernel in front whatever the size
         _check(values, segs, op, init, oracle, name)
+        _check(values, segs, op, init, oracle, name + "/partitioned", phases=7 | 8)
 
 
 def test_float_specials(dev, oracle):
@@ -163,8 +166,9 @@ def test_spine_levels(dev, oracle):
     values = rng.integers(-1000, 1000, size=count).astype(np.int32)
     for segs in ([0], [0, 5], [0, nv - 1], [0, nv - 1, 1030 * nv - 1030, 2000 * nv],
                  [0, 0, 0, count - 1, count, count]):
-        _check(values, np.array(segs, dtype=np.int32), "plus", -3, oracle, str(segs))
-        _check(values, np.array(segs, dtype=np.int32), "maximum", -3, oracle, str(segs))
+        for phases in (7, 7 | 8):       # own splits, and the partition kernel
+            _check(values, np.array(segs, dtype=np.int32), "plus", -3, oracle, str(segs), phases)
+            _check(values, np.array(segs, dtype=np.int32), "maximum", -3, oracle, str(segs), phases)
 
 
 @pytest.mark.parametrize("tiles", [4096, 4097])
