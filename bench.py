@@ -690,9 +690,14 @@ def cpu_baseline(wk, budget_s, all_cores):
 
 
 # BASELINE.json's configs beside the headline one (configs[1]): configs[0],
-# both halves of configs[2], configs[3], both halves of configs[4].
+# both halves of configs[2], configs[3], both halves of configs[4]; then the
+# steps on either side of the path (scan, reduce, lbs_segreduce, the interval
+# moves, work creation, sorted search and join).  About 50 s in all.
 DEFAULT_EXTRA = ("c1_segreduce_i32,c3_load_balance_search,c3_interval_expand_i32,"
-                 "c4_spmv_f32,c5_f64max,c5_i64sum")
+                 "c4_spmv_f32,c5_f64max,c5_i64sum,"
+                 "scan_i32,reduce_f32,c2_lbs_segreduce_i32,c3_interval_gather_i32,"
+                 "c3_interval_scatter_i32,c3_interval_move_i32,workcreate_i32,"
+                 "sorted_search_i32,inner_join_i32")
 
 
 def main():
@@ -787,7 +792,14 @@ def main():
     main_res = measure(args.workload, True)
     others = {}
     for key in [k for k in args.extra.split(",") if k and k != args.workload]:
-        r = measure(key, False)
+        # A further workload that fails (its parity check included) is
+        # reported as failed; it does not take the headline with it.
+        try:
+            r = measure(key, False)
+        except (Exception, SystemExit) as e:
+            others[key] = {"error": str(e) or type(e).__name__}
+            torch.cuda.empty_cache()
+            continue
         others[key] = {k: r[k] for k in (
             "description", "dtype", "ms_per_step", "median_ms_per_step", "GBps", "items_per_s",
             "pct_hbm_peak", "pct_hbm_peak_median", "algorithmic_bytes", "roofline")}
