@@ -188,7 +188,7 @@ def make_c3_moves(copies, kind):
     wk.key = "c3_interval_%s_i32" % kind
     wk.name = "interval_%s int32, 2^24 Zipf(1.2) segments, 2^28 items, segments placed " \
               "in random order" % kind
-    wk.kernel = "transform_lbs_f<512x12, %s> (whole call)" % kind
+    wk.kernel = "partition + transform_lbs_f<512x16, %s> (whole call)" % kind
     wk.bytes = n * 4 + n * 4 + s * 4 + s * 4 * (2 if kind == "move" else 1)
     if kind == "gather":
         wk.step = lambda i: m.interval_gather(inps[i % copies], n, segs[i % copies],
