@@ -261,8 +261,70 @@ static int check_box(context_t& context) {
   return 0;
 }
 
+// Segments that span hundreds of tiles under operators that do not commute:
+// the carries of such a segment are folded by the spine in a loop of its own
+// (rows of consecutive carries per wavefront, several wavefronts), and any
+// carry taken out of order shows.  Affine maps x -> a x + b composed left to
+// right, packed in 4 bytes (mod 2^16) and in 8 bytes (mod 2^32), and the
+// 16-byte matrices above.
+struct affine16_mul_t {
+  MGPU_HOST_DEVICE unsigned operator()(unsigned f, unsigned g) const {
+    unsigned fa = f >> 16, fb = f & 0xffff, ga = g >> 16, gb = g & 0xffff;
+    return ((fa * ga) & 0xffff) << 16 | ((ga * fb + gb) & 0xffff);
+  }
+};
+struct affine32_t {
+  unsigned a, b;
+  MGPU_HOST_DEVICE bool operator==(const affine32_t& r) const {
+    return a == r.a && b == r.b;
+  }
+};
+struct affine32_mul_t {
+  MGPU_HOST_DEVICE affine32_t operator()(affine32_t f, affine32_t g) const {
+    return affine32_t { f.a * g.a, g.a * f.b + g.b };
+  }
+};
+
+template<typename type_t, typename op_t, typename make_t>
+static int check_long_runs_of(make_t make, op_t op, type_t init,
+  context_t& context) {
+  const int counts[] = { 9000001, 2000003, 777777 };
+  const int begins[] = { 5, 4099, 70001 };
+  for(int count : counts) for(int begin : begins) {
+    // An empty segment, a short one, the long one, a short tail.
+    std::vector<int> seg_host = { 0, 0, begin, count - 7 };
+    int num_segments = (int)seg_host.size();
+    mem_t<int> segments = to_mem(seg_host, context);
+    mem_t<type_t> results(num_segments, context);
+    transform_segreduce(make, count, segments.data(), num_segments,
+      results.data(), op, init, context);
+    std::vector<type_t> got = from_mem(results);
+    for(int s = 0; s < num_segments; ++s) {
+      int b = seg_host[s], e = s + 1 < num_segments ? seg_host[s + 1] : count;
+      type_t want = init;
+      for(int i = b; i < e; ++i) want = (i == b) ? make(i) : op(want, make(i));
+      CHECK(got[s] == want);
+    }
+  }
+  return 0;
+}
+
+static int check_long_runs(context_t& context) {
+  CHECK(0 == check_long_runs_of<unsigned>([] __host__ __device__ (int i) {
+    return (unsigned)((1 + 2 * (i % 7)) << 16 | (i % 11));
+  }, affine16_mul_t(), 0x10000u, context));
+  CHECK(0 == check_long_runs_of<affine32_t>([] __host__ __device__ (int i) {
+    return affine32_t { 1u + 2 * ((unsigned)i % 5), (unsigned)i % 13 };
+  }, affine32_mul_t(), affine32_t { 1, 0 }, context));
+  CHECK(0 == check_long_runs_of<mat_t>([] __host__ __device__ (int i) {
+    return mat_of(i);
+  }, mat_mul_t(), mat_t { 9, 9, 9, 9 }, context));
+  return 0;
+}
+
 int main() {
   standard_context_t context(false);
+  CHECK(0 == check_long_runs(context));
   CHECK(0 == (check_box<launch_params_t<64, 1> >(context)));
   CHECK(0 == (check_box<launch_params_t<64, 3> >(context)));
   CHECK(0 == (check_box<launch_params_t<128, 7> >(context)));
