@@ -915,14 +915,17 @@ struct cached_segment_load_t {
   enum { size = tuple_size<pointers_t>::value };
   typedef tuple_iterator_value_t<pointers_t> value_t;
 
-  // Values of up to 8 bytes are staged for up to 2 * nt - 32 segments (two
+  // Values of up to 16 bytes are staged for up to 2 * nt - 32 segments (two
   // reads per thread), wider ones for up to nt: a tile of 512 x 16 elements
   // can begin 873 segments on the 2^24-segment benchmark input, and a tile
   // with more segments than are staged has every item gather its own value
   // from global memory, which costs several times what staging does.
+  // Values of up to 8 bytes are all read ahead by fetch(); of wider ones
+  // only the first row is (registers), and commit() reads the second.
   enum {
-    rows = sizeof(value_t) <= 8 ? 2 : 1,
-    capacity = rows * nt - (rows > 1 ? 32 : 0)
+    staged_rows = sizeof(value_t) <= 16 ? 2 : 1,
+    rows = sizeof(value_t) <= 8 ? staged_rows : 1,
+    capacity = staged_rows * nt - (staged_rows > 1 ? 32 : 0)
   };
   struct storage_t {
     value_t data[capacity];
@@ -939,7 +942,7 @@ struct cached_segment_load_t {
     storage_t& storage, pointers_t iterators) {
     fetched_t x;
     bool fits = fetch(tid, begin, count, iterators, x);
-    commit(tid, begin, count, x, storage);
+    commit(tid, begin, count, x, storage, iterators);
     return fits;
   }
   // The same in two steps, so that the global read can be in flight while
@@ -958,12 +961,22 @@ struct cached_segment_load_t {
     return true;
   }
   MGPU_DEVICE static void commit(int tid, int begin, int count,
-    const fetched_t& fetched, storage_t& storage) {
+    const fetched_t& fetched, storage_t& storage, pointers_t iterators) {
     if(count > capacity) return;
+    // Rows that fetch() has not read ahead.
+    value_t late[staged_rows - rows + 1];
     PRAGMA_UNROLL
-    for(int r = 0; r < rows; ++r) {
+    for(int r = rows; r < staged_rows; ++r) {
       int at = nt * r + tid;
-      if(at < count && begin + at >= 0) storage.data[at] = fetched.x[r];
+      if(at < count && begin + at >= 0)
+        late[r - rows] = mgpu::load(iterators, begin + at);
+    }
+    PRAGMA_UNROLL
+    for(int r = 0; r < staged_rows; ++r) {
+      int at = nt * r + tid;
+      if(at < count && begin + at >= 0)
+        storage.data[at] = r < rows ? fetched.x[r < rows ? r : 0] :
+          late[r < rows ? 0 : r - rows];
     }
     __syncthreads();
   }
@@ -1010,7 +1023,7 @@ struct cached_segment_load_t<nt, tuple<> > {
     return false;
   }
   MGPU_DEVICE static void commit(int, int, int, const fetched_t&,
-    storage_t&) {
+    storage_t&, tuple<>) {
   }
   MGPU_DEVICE static value_t get(bool, int, int, const storage_t&, tuple<>) {
     return value_t();

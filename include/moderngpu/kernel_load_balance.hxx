@@ -165,7 +165,7 @@ struct transform_lbs_f {
         load_balance_t().fill_compact(range, segments, tid, shared.lbs,
           ahead[g]);
       cached_load_t::commit(tid, seg_base, range.b_count() + 1, fetched[g],
-        shared.cached);
+        shared.cached, caching_iterators);
       const typename load_balance_t::slot_t* slots = tile.slots;
 
       // The emission loop exists twice -- cached values staged in LDS, or

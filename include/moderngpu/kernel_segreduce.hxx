@@ -350,7 +350,7 @@ struct segreduce_tile_f {
         input.caching_iterators, fetched);
       load_balance_t().fill(range, segments, tid, shared.source.lbs);
       cached_load_t::commit(tid, seg_base, range.b_count() + 1, fetched,
-        shared.source.cached);
+        shared.source.cached, input.caching_iterators);
       const int* slots = shared.source.lbs.indices;
       const int* starts = slots + load_balance_t::starts_offset(a_count);
       PRAGMA_UNROLL

@@ -116,7 +116,7 @@ struct workcreate_tile_t {
       range.b_count() + 1, caching_iterators, fetched);
     load_balance_t().fill(range, segments, tid, shared.lbs, ahead);
     cached_load_t::commit(tid, range.b_begin - 1, range.b_count() + 1,
-      fetched, shared.cached);
+      fetched, shared.cached, caching_iterators);
     return decoded_t { range, staged };
   }
 

@@ -51,13 +51,16 @@ typedef detail::lbs_store_seg_f<int*> store_seg_f;
 template<typename type_t>
 using expand_f = detail::interval_expand_f<type_t, type_t*>;
 // gather / scatter / move: the library's own pointer functors (W consecutive
-// items per call).
+// items per call for elements of less than 16 bytes).
 template<typename type_t>
-using gather_f = detail::interval_copy_chunks_f<false, true, type_t>;
+using gather_f = typename detail::interval_copy_select_t<false, true,
+  const type_t*, type_t*>::type;
 template<typename type_t>
-using scatter_f = detail::interval_copy_chunks_f<true, false, type_t>;
+using scatter_f = typename detail::interval_copy_select_t<true, false,
+  const type_t*, type_t*>::type;
 template<typename type_t>
-using move_f = detail::interval_copy_chunks_f<true, true, type_t>;
+using move_f = typename detail::interval_copy_select_t<true, true,
+  const type_t*, type_t*>::type;
 
 template<int bytes>
 int expand_sized(const void* input, int count, const int* segments,
