@@ -446,6 +446,60 @@ def make_c5(copies, kind):
     return wk
 
 
+def make_c2_typed(copies, dtype_name, op):
+    """segreduce on the C2 segments for any of the library's value types and
+    operators (the headline workload is float32 plus): integer results must
+    equal the CPU loop's, floating ones must lie within 1e-5 (float32) or 1e-12
+    (float64) of it, relative to the sum of the segment's magnitudes."""
+    import torch
+    import moderngpu_amd as m
+    from moderngpu_amd import workloads
+    from oracle import oracle
+    np_type = {"i32": np.int32, "u32": np.uint32, "f32": np.float32,
+               "i64": np.int64, "u64": np.uint64, "f64": np.float64}[dtype_name]
+    unsigned = dtype_name in ("u32", "u64")
+    copies = min(copies, 3)
+    count, starts = workloads.config2_segments()
+    s = starts.size
+    rng = np.random.Generator(np.random.PCG64(7))
+    if np.dtype(np_type).kind == "f":
+        host = [rng.random(count, dtype=np_type) for _ in range(copies)]
+    else:
+        host = [rng.integers(0, 1 << 20, size=count, dtype=np.int64).astype(np_type)
+                for _ in range(copies)]
+    as_signed = {np.uint32: np.int32, np.uint64: np.int64}
+    vals = [_dev(h.view(as_signed[np_type]) if unsigned else h) for h in host]
+    segs = [_dev(starts) for _ in range(copies)]
+    outs = [torch.empty(s, dtype=vals[0].dtype, device="cuda") for _ in range(copies)]
+    size = host[0].itemsize
+    wk = Workload()
+    wk.key = "c2_segreduce_%s_%s" % (dtype_name, op)
+    wk.name = "segreduce %s %s, 2^26 values, 2^20 geometric segments" % (dtype_name, op)
+    wk.dtype, wk.items = dtype_name, count
+    wk.bytes = count * size + s * 4 + s * size
+    wk.kernel = "segreduce_tile_f<%s, %s>" % (dtype_name, op)
+    calls = [m.prepare_segreduce(vals[c], segs[c], op, 0, out=outs[c], unsigned=unsigned)[0]
+             for c in range(copies)]
+    tiles = [m.prepare_segreduce(vals[c], segs[c], op, 0, out=outs[c], unsigned=unsigned,
+                                 phases=2)[0] for c in range(copies)]
+    wk.step = lambda i: calls[i % copies]()
+    wk.tiles = lambda i: tiles[i % copies]()
+
+    def check():
+        got = calls[0]().cpu().numpy()
+        got = got.view(np_type) if unsigned else got
+        want = oracle.segreduce(host[0], starts, op, 0)
+        if np.dtype(np_type).kind != "f":
+            return bool(np.array_equal(got, want))
+        tol = 1e-5 if np_type == np.float32 else 1e-12
+        # the values are not negative: |want| is the sum of magnitudes
+        return bool(np.all(np.abs(got.astype(np.float64) - want.astype(np.float64))
+                           <= tol * np.abs(want) + 1e-300))
+    wk.check = check
+    wk.cpu = lambda: (lambda: oracle.segreduce(host[0], starts, op, 0))
+    return wk
+
+
 def make_c1(copies):
     import torch
     import moderngpu_amd as m
@@ -584,6 +638,12 @@ FACTORIES = {
     "c5_f64max": lambda c: make_c5(c, "f64max"),
     "c5_i64sum": lambda c: make_c5(c, "i64sum"),
 }
+
+for _t in ("i32", "u32", "f32", "i64", "u64", "f64"):
+    for _op in ("plus", "maximum", "minimum"):
+        FACTORIES["c2_segreduce_%s_%s" % (_t, _op)] = \
+            (lambda t, o: lambda c: make_c2_typed(c, t, o))(_t, _op)
+
 
 def traffic_table():
     """HBM bytes per launch of each workload's dominant kernel, from the table
