@@ -44,6 +44,17 @@ using namespace mgpu::detail;
 // resident CTAs per CU matter more here than the longest possible tile.
 typedef launch_box_t<arch_gfx950_cta<256, 12, 12> > workcreate_launch_default_t;
 
+// An upsweep functor that looks at nothing but the item's index may say so:
+//   typedef void index_only_tag;
+// Its tiles are then not decoded in the upsweep (segment, rank and cached
+// values of its calls are meaningless): 2^26 items 67 -> 62 us.
+template<typename func_t, typename enable_t = void>
+struct is_index_only_t : std::false_type { };
+template<typename func_t>
+struct is_index_only_t<func_t,
+  typename std::conditional<false, typename func_t::index_only_tag,
+    void>::type> : std::true_type { };
+
 template<typename arg_t>
 struct is_tuple_t : std::false_type { };
 template<typename... args_t>
@@ -207,7 +218,12 @@ struct workcreate_upsweep_f {
     int tile = xcd_tile(cta, tiles.num_tiles);
     if(tile >= tiles.num_tiles) return;
     __shared__ typename tile_t::storage_t shared;
-    typename tile_t::decoded_t decoded = tiles.decode(tid, tile, shared);
+    typename tile_t::decoded_t decoded;
+    if constexpr(is_index_only_t<func_t>::value)
+      decoded.range = paired_tile_range(tiles.count, tiles.num_segments, tile,
+        tile_t::load_balance_t::nv, tiles.pairs);
+    else
+      decoded = tiles.decode(tid, tile, shared);
 
     // Bit i: item nt * i + tid exists.
     int a_count = decoded.range.a_count();
@@ -216,7 +232,13 @@ struct workcreate_upsweep_f {
     for(int i = 0; i < vt; ++i)
       valid |= (unsigned)(nt * i + tid < a_count) << i;
     typename tile_t::items_t x;
-    tiles.items(tid, decoded, shared, valid, x);
+    if constexpr(is_index_only_t<func_t>::value) {
+      PRAGMA_UNROLL
+      for(int i = 0; i < vt; ++i) {
+        x.seg[i] = 0; x.rank[i] = 0; x.cached[i] = value_t();
+      }
+    } else
+      tiles.items(tid, decoded, shared, valid, x);
 
     // All calls first, their results -- which usually come from memory --
     // are only looked at afterwards, so the loads of all calls overlap.

@@ -46,6 +46,7 @@ struct workspace_t {
 };
 
 struct created_f {
+  typedef void index_only_tag;      // the upsweep need not decode its tiles
   const int* created;
   MGPU_DEVICE int operator()(int index, int, int, tuple<>) const {
     return created[index];
