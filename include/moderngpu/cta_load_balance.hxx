@@ -156,8 +156,11 @@ MGPU_DEVICE inline merge_range_t paired_tile_range(int count,
   int a1 = pairs[2 * tile + 2], b1 = pairs[2 * tile + 3];
   a0 = min(max(a0, 0), count);
   b0 = min(max(b0, 0), num_segments);
-  a1 = min(a0 + min(max(a1 - a0, 0), nv), count);
-  b1 = min(b0 + min(max(b1 - b0, 0), nv - (a1 - a0)), num_segments);
+  // (unsigned: a0 + nv may pass 2^31 when count is close to the index limit)
+  a1 = (int)min(min((unsigned)max(a1, a0), (unsigned)a0 + (unsigned)nv),
+    (unsigned)count);
+  b1 = (int)min(min((unsigned)max(b1, b0),
+    (unsigned)b0 + (unsigned)(nv - (a1 - a0))), (unsigned)num_segments);
   return merge_range_t { a0, a1, b0, b1 };
 }
 
