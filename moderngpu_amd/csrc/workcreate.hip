@@ -48,8 +48,10 @@ struct workspace_t {
 struct created_f {
   typedef void index_only_tag;      // the upsweep need not decode its tiles
   const int* created;
+  // The counts are streamed once per sweep: non-temporal loads (2^26 items:
+  // whole call 230 -> 219 us).
   MGPU_DEVICE int operator()(int index, int, int, tuple<>) const {
-    return created[index];
+    return __builtin_nontemporal_load(created + index);
   }
 };
 
@@ -64,7 +66,7 @@ struct record_f {
     if(source_index) source_index[dest_seg] = index;
     if(source_seg) source_seg[dest_seg] = seg;
     if(source_rank) source_rank[dest_seg] = rank;
-    return created[index];
+    return __builtin_nontemporal_load(created + index);
   }
 };
 
