@@ -39,7 +39,7 @@ static int test_seg_plus_rank(int count, int num_segments, int seed,
     int end = (seg + 1 < num_segments) ? segments_host[seg + 1] : count;
     int x = init;
     for(int rank = 0; rank < end - begin; ++rank)
-      x = rank ? x + seg + rank : seg + rank;
+      x = rank ? (int)((unsigned)x + (unsigned)(seg + rank)) : seg + rank;   // wraps like the device sum
     CHECK(x == results_host[seg], "seed %d segment %d [%d, %d): device %d host %d",
       seed, seg, begin, end, results_host[seg], x);
   }
