@@ -126,7 +126,12 @@ struct lane_words_t {
 };
 
 // v_mov_b32_dpp per 32-bit word.  Lanes with no source (outside the row for
-// row_shr, outside row_mask for the broadcasts) keep `old`.
+// row_shr, outside row_mask for the broadcasts) keep `old` -- and so does a
+// lane whose source lane is switched off.  Every cross-lane helper below
+// therefore has to be called by all lanes whose values may be read: never
+// behind a lane-dependent branch, and not on the right of `||`, `&&` or `?:`
+// either (`!lane || wave_shift_up1(x) != x` runs the shift with lane 0 off,
+// and lane 1 then compares x with itself).
 template<int ctrl, int row_mask = 0xf, int bank_mask = 0xf, typename type_t>
 MGPU_DEVICE inline type_t dpp_move(type_t old, type_t src) {
   lane_words_t<type_t> o(old), s(src);
