@@ -500,6 +500,120 @@ def make_c2_typed(copies, dtype_name, op):
     return wk
 
 
+def make_shape(copies, spec):
+    """Workloads of a given shape, for looking at the library outside the
+    BASELINE configurations: --workload shape:<op>:<log2 items>:<segments>
+      op        segreduce (float32 plus) | lbs (load_balance_search) |
+                expand<bytes> (interval_expand of 1/2/4/8/16-byte elements)
+      segments  len<k>   every segment k items long
+                nseg<k>  k segments, starts drawn uniformly (sorted)
+    e.g. shape:segreduce:26:nseg1024, shape:lbs:20:len16, shape:expand16:28:len16.
+    Parity: segreduce against float64 sums (1e-5 of the sum of magnitudes), lbs
+    and expand against numpy."""
+    import torch
+    import moderngpu_amd as m
+    from oracle import oracle
+    _, op, log2n, segspec = spec.split(":")
+    n = 1 << int(log2n)
+    rng = np.random.Generator(np.random.PCG64(11))
+    if segspec.startswith("len"):
+        starts = np.arange(0, n, int(segspec[3:]), dtype=np.int64)
+    elif segspec.startswith("nseg"):
+        k = int(segspec[4:])
+        starts = np.concatenate([[0], np.sort(rng.integers(0, n, size=k - 1))])
+    else:
+        raise ValueError("segments: len<k> or nseg<k>")
+    starts = starts.astype(np.int32)
+    s = starts.size
+    copies = min(copies, 3)
+    segs = _dev(starts)
+    wk = Workload()
+    wk.key, wk.items = spec, n
+    wk.kernel = "whole call"
+    if op == "segreduce":
+        host = [rng.random(n, dtype=np.float32) for _ in range(copies)]
+        vals = [_dev(h) for h in host]
+        out = torch.empty(s, dtype=torch.float32, device="cuda")
+        calls = [m.prepare_segreduce(v, segs, "plus", 0.0, out=out)[0] for v in vals]
+        tiles = [m.prepare_segreduce(v, segs, "plus", 0.0, out=out, phases=2)[0] for v in vals]
+        wk.dtype, wk.bytes = "f32", n * 4 + s * 4 + s * 4
+        wk.name = "segreduce float32 plus, 2^%s values, %d segments (%s)" % (log2n, s, segspec)
+        wk.step = lambda i: calls[i % copies]()
+        wk.tiles = lambda i: tiles[i % copies]()
+        wk.kernel = "segreduce_tile_f<256x16, float, plus>"
+
+        def check():
+            # float64 sums of the same values (they are not negative, so the
+            # sum is also the sum of magnitudes the tolerance is relative to)
+            got = calls[0]().cpu().numpy().astype(np.float64)
+            c = np.concatenate([[0.0], np.cumsum(host[0], dtype=np.float64)])
+            ends = np.append(starts[1:], n).astype(np.int64)
+            want = c[ends] - c[starts.astype(np.int64)]
+            return bool(np.all(np.abs(got - want) <= 1e-5 * np.abs(want) + 1e-30))
+        wk.check = check
+        wk.cpu = lambda: (lambda: oracle.segreduce(host[0], starts, "plus", 0.0))
+    elif op == "lbs":
+        outs = [torch.empty(n, dtype=torch.int32, device="cuda") for _ in range(copies)]
+        calls = [m.prepare_load_balance_search(n, segs, out=o)[0] for o in outs]
+        wk.dtype, wk.bytes = "i32", n * 4 + s * 4
+        wk.name = "load_balance_search, 2^%s items, %d segments (%s)" % (log2n, s, segspec)
+        wk.step = lambda i: calls[i % copies]()
+        wk.tiles = wk.step
+        want = lambda: (np.searchsorted(starts, np.arange(n, dtype=np.int32), side="right")
+                        - 1).astype(np.int32)
+        wk.check = lambda: bool(np.array_equal(wk.step(0).cpu().numpy(), want()))
+        wk.cpu = lambda: (lambda: oracle.load_balance_search(n, starts))
+    elif op.startswith("expand"):
+        size = int(op[6:])
+        words = max(size // 8, 1)
+        np_type = {1: np.uint8, 2: np.int16, 4: np.int32}.get(size, np.int64)
+        host = rng.integers(0, 100, size=(s, words) if size == 16 else s).astype(np_type)
+        vals = _dev(host)
+        if size == 16:
+            vals = vals.view(torch.complex128).reshape(s)
+        outs = [torch.empty(n, dtype=vals.dtype, device="cuda") for _ in range(min(copies, 2))]
+        wk.dtype, wk.bytes = "%d-byte" % size, n * size + s * 4 + s * size
+        wk.name = "interval_expand of %d-byte elements, 2^%s items, %d segments (%s)" % (
+            size, log2n, s, segspec)
+        wk.step = lambda i: m.interval_expand(vals, n, segs, out=outs[i % len(outs)])
+        wk.tiles = wk.step
+
+        def check():
+            got = wk.step(0)
+            if size == 16:
+                got = got.view(torch.float64).view(torch.int64).reshape(n, 2)
+            lens = np.diff(np.append(starts.astype(np.int64), n))
+            return bool(np.array_equal(got.cpu().numpy(), np.repeat(host, lens, axis=0)))
+        wk.check = check
+        wk.cpu = lambda: (lambda: np.repeat(host, np.diff(np.append(starts.astype(np.int64), n)),
+                                            axis=0))
+    else:
+        raise ValueError("op: segreduce, lbs or expand<bytes>")
+    return wk
+
+
+def make_cumsum_probe(copies):
+    """Not a kernel of this library: torch.cumsum over 2^26 int32, the
+    single-pass scan the platform's library offers, beside scan_i32."""
+    import torch
+    n = 1 << 26
+    rng = np.random.Generator(np.random.PCG64(42))
+    host = rng.integers(0, 128, size=n, dtype=np.int32)
+    xs = [_dev(host) for _ in range(copies)]
+    outs = [torch.empty(n, dtype=torch.int32, device="cuda") for _ in range(copies)]
+    wk = Workload()
+    wk.key, wk.dtype, wk.items = "scan_probe_torch_cumsum_i32", "i32", n
+    wk.name = "torch.cumsum (inclusive), 2^26 int32"
+    wk.bytes = n * 4 + n * 4
+    wk.kernel = "torch cumsum (yardstick, not part of the library)"
+    wk.step = lambda i: torch.cumsum(xs[i % copies], 0, dtype=torch.int32, out=outs[i % copies])
+    wk.tiles = wk.step
+    wk.check = lambda: bool(np.array_equal(wk.step(0).cpu().numpy(),
+                                           np.cumsum(host, dtype=np.int32)))
+    wk.cpu = lambda: (lambda: np.cumsum(host, dtype=np.int32))
+    return wk
+
+
 def make_c1(copies):
     import torch
     import moderngpu_amd as m
@@ -628,6 +742,7 @@ FACTORIES = {
     "inner_join_i32": lambda c: make_search(c, "join"),
     "c4_spmv_f32": make_c4,
     "c4_gather_probe_f32": make_c4_gather_probe,
+    "scan_probe_torch_cumsum_i32": make_cumsum_probe,
     "store_probe_linear_read0": lambda c: make_store_probe(c, 0, 0),
     "store_probe_runs_read0": lambda c: make_store_probe(c, 1, 0),
     "store_probe_eighths_read0": lambda c: make_store_probe(c, 2, 0),
@@ -765,7 +880,9 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=30)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="c2_segreduce_f32", choices=sorted(FACTORIES))
+    ap.add_argument("--workload", default="c2_segreduce_f32",
+                    help="one of %s, or shape:<op>:<log2 items>:<segments> (see make_shape)"
+                    % ", ".join(sorted(FACTORIES)))
     ap.add_argument("--copies", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--extra", default=DEFAULT_EXTRA,
@@ -804,7 +921,12 @@ def main():
     traffic = traffic_table()
 
     def measure(key, headline):
-        wk = FACTORIES[key](args.copies)
+        if key.startswith("shape:"):
+            wk = make_shape(args.copies, key)
+        elif key in FACTORIES:
+            wk = FACTORIES[key](args.copies)
+        else:
+            sys.exit("unknown workload %s" % key)
         if not wk.check():
             sys.exit("parity check failed for %s: no throughput reported" % key)
         # The contract's figure: exactly `steps` steps between two
