@@ -504,7 +504,9 @@ def make_shape(copies, spec):
     """Workloads of a given shape, for looking at the library outside the
     BASELINE configurations: --workload shape:<op>:<log2 items>:<segments>
       op        segreduce (float32 plus) | lbs (load_balance_search) |
-                expand<bytes> (interval_expand of 1/2/4/8/16-byte elements)
+                expand<bytes> (interval_expand of 1/2/4/8/16-byte elements) |
+                gather<bytes>, scatter<bytes>, move<bytes> (the interval moves
+                with every segment in place)
       segments  len<k>   every segment k items long
                 nseg<k>  k segments, starts drawn uniformly (sorted)
     e.g. shape:segreduce:26:nseg1024, shape:lbs:20:len16, shape:expand16:28:len16.
@@ -587,8 +589,34 @@ def make_shape(copies, spec):
         wk.check = check
         wk.cpu = lambda: (lambda: np.repeat(host, np.diff(np.append(starts.astype(np.int64), n)),
                                             axis=0))
+    elif op[:6] in ("gather", "scatte") or op.startswith("move"):
+        # interval_gather / _scatter / _move with every segment in place
+        # (its base is its own start): the output equals the input.
+        kind = "gather" if op.startswith("gather") else (
+            "scatter" if op.startswith("scatter") else "move")
+        size = int(op[len(kind):])
+        host = rng.integers(0, 1 << 30, size=(n, 2) if size == 16 else n).astype(
+            {1: np.uint8, 2: np.int16, 4: np.int32}.get(size, np.int64))
+        inp = _dev(host)
+        if size == 16:
+            inp = inp.view(torch.complex128).reshape(n)
+        out = torch.empty_like(inp)
+        wk.dtype, wk.bytes = "%d-byte" % size, 2 * n * size + 2 * s * 4
+        wk.name = "interval_%s of %d-byte elements, 2^%s items, %d segments in place (%s)" % (
+            kind, size, log2n, s, segspec)
+        if kind == "gather":
+            wk.step = lambda i: m.interval_gather(inp, n, segs, segs, out=out)
+        elif kind == "scatter":
+            wk.step = lambda i: m.interval_scatter(inp, n, segs, segs, out)
+        else:
+            wk.step = lambda i: m.interval_move(inp, n, segs, segs, segs, out)
+        wk.tiles = wk.step
+        as_ints = lambda t: t.view(torch.float64).view(torch.int64) if size == 16 else t
+        wk.check = lambda: bool(torch.equal(as_ints(wk.step(0)), as_ints(inp)))
+        wk.cpu = lambda: (lambda: host.copy())
     else:
-        raise ValueError("op: segreduce, lbs or expand<bytes>")
+        raise ValueError("op: segreduce, lbs, expand<bytes>, gather<bytes>, scatter<bytes> "
+                         "or move<bytes>")
     return wk
 
 
