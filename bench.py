@@ -119,7 +119,7 @@ def make_c3(copies, expand=False):
         wk.key = "c3_interval_expand_i32"
         wk.name = "interval_expand int32, 2^24 Zipf(1.2) segments, 2^28 items"
         wk.bytes = s * 4 + s * 4 + n * 4
-        wk.kernel = "transform_lbs_f<512x12, expand>"
+        wk.kernel = "transform_lbs_f<512x16, expand>"
         wk.step = lambda i: m.interval_expand(vals[i % copies], n, segs[i % copies],
                                               out=outs[i % copies])
         wk.tiles = lambda i: m.interval_expand(vals[i % copies], n, segs[i % copies],
@@ -188,7 +188,7 @@ def make_c3_moves(copies, kind):
     wk.key = "c3_interval_%s_i32" % kind
     wk.name = "interval_%s int32, 2^24 Zipf(1.2) segments, 2^28 items, segments placed " \
               "in random order" % kind
-    wk.kernel = "partition + transform_lbs_f<512x16, %s> (whole call)" % kind
+    wk.kernel = "partition + transform_lbs_f<512x16, %s>" % kind
     wk.bytes = n * 4 + n * 4 + s * 4 + s * 4 * (2 if kind == "move" else 1)
     if kind == "gather":
         wk.step = lambda i: m.interval_gather(inps[i % copies], n, segs[i % copies],
@@ -227,7 +227,7 @@ def make_lbs_segreduce(copies):
     wk.dtype, wk.items = "i32", n
     wk.key = "c2_lbs_segreduce_i32"
     wk.name = "lbs_segreduce f = seg + rank, int32 plus, 2^26 computed items, 2^20 segments"
-    wk.kernel = "segreduce_tile_f<lbs input> + partition + spine (whole call)"
+    wk.kernel = "partition + segreduce_tile_f<lbs input> + spine"
     wk.bytes = s * 4 + s * 4
     wk.step = lambda i: m.lbs_segreduce_seg_plus_rank(n, segs[i % copies], -1,
                                                       out=outs[i % copies])
@@ -258,7 +258,7 @@ def make_search(copies, kind):
         wk.key, wk.items = "sorted_search_i32", n
         wk.name = "sorted_search lower bound, 2^26 needles in 2^26 haystack keys"
         wk.bytes = n * 4 + h * 4 + n * 4
-        wk.kernel = "merge_path_partition_f + sorted_search_f<256x12> (whole call)"
+        wk.kernel = "partition + sorted_search_f<256x12>"
         wk.step = lambda i: m.sorted_search(dn[i % copies], dh[i % copies], "lower",
                                             out=outs[i % copies])
         wk.check = lambda: bool(np.array_equal(
@@ -274,7 +274,7 @@ def make_search(copies, kind):
         wk.key, wk.items = "inner_join_i32", 2 * n
         wk.name = "inner_join, 2^24 keys a side, %d pairs" % pairs
         wk.bytes = 2 * n * 4 + pairs * 8
-        wk.kernel = "2 x sorted_search + scan + transform_lbs (whole call, one host wait)"
+        wk.kernel = "sorted_search (lower + counts) + scan + transform_lbs"
         wk.step = lambda i: m.inner_join(da[i % copies], db[i % copies])
         wk.check = lambda: bool(np.array_equal(wk.step(0).cpu().numpy(),
                                                oracle.inner_join(a, b)))
@@ -689,7 +689,7 @@ def make_scan(copies, kind):
         wk.key, wk.dtype = "scan_i32", "i32"
         wk.name = "exclusive plus-scan, 2^26 int32 (segment lengths -> starts)"
         wk.bytes = n * 4 + n * 4
-        wk.kernel = "scan upsweep + spine + downsweep (whole call)"
+        wk.kernel = "scan upsweep + spine + downsweep"
         wk.step = lambda i: m.scan(vals[i % copies], "plus", out=outs[i % copies],
                                    reduction=red)[0]
         wk.tiles = wk.step
@@ -704,7 +704,7 @@ def make_scan(copies, kind):
         wk.key, wk.dtype = "reduce_f32", "f32"
         wk.name = "plus-reduce, 2^26 float32"
         wk.bytes = n * 4
-        wk.kernel = "scan_upsweep_f + reduce_final_f (whole call)"
+        wk.kernel = "scan_upsweep_f + reduce_final_f"
         wk.step = lambda i: m.reduce(vals[i % copies], "plus", out=out)
         wk.tiles = wk.step
 
@@ -740,7 +740,7 @@ def make_workcreate(copies):
     # upsweep: counts + starts in; downsweep: starts + the creators' counts in,
     # four ints per new segment out.
     wk.bytes = n * 4 + s * 4 + s * 4 + k * 4 + k * 16
-    wk.kernel = "workcreate upsweep + totals scan + downsweep (whole call, one host wait)"
+    wk.kernel = "workcreate upsweep + scan + downsweep"
     wk.step = lambda i: m.workcreate(created[i % copies], segs[i % copies])
     wk.tiles = wk.step
 
@@ -906,15 +906,153 @@ def cpu_baseline(wk, budget_s, all_cores):
     return res
 
 
-# BASELINE.json's configs beside the headline one (configs[1]): configs[0],
-# both halves of configs[2], configs[3], both halves of configs[4]; then the
-# steps on either side of the path (scan, reduce, lbs_segreduce, the interval
-# moves, work creation, sorted search and join).  About 50 s in all.
-DEFAULT_EXTRA = ("c1_segreduce_i32,c3_load_balance_search,c3_interval_expand_i32,"
-                 "c4_spmv_f32,c5_f64max,c5_i64sum,"
-                 "scan_i32,reduce_f32,c2_lbs_segreduce_i32,c3_interval_gather_i32,"
-                 "c3_interval_scatter_i32,c3_interval_move_i32,workcreate_i32,"
-                 "sorted_search_i32,inner_join_i32")
+# Reported under 'others' in this order: first the steps on either side of the
+# path (scan, reduce, lbs_segreduce, the interval moves, work creation, sorted
+# search and join), then BASELINE.json's configs beside the headline one
+# (configs[1]): configs[0], both halves of configs[2], configs[3], both halves
+# of configs[4].  Whoever keeps only the end of the line keeps those.  About
+# 55 s in all.
+BASELINE_EXTRA = ("c1_segreduce_i32", "c3_load_balance_search", "c3_interval_expand_i32",
+                  "c4_spmv_f32", "c5_f64max", "c5_i64sum")
+DEFAULT_EXTRA = ",".join(("scan_i32", "reduce_f32", "c2_lbs_segreduce_i32",
+                          "c3_interval_gather_i32", "c3_interval_scatter_i32",
+                          "c3_interval_move_i32", "workcreate_i32", "sorted_search_i32",
+                          "inner_join_i32") + BASELINE_EXTRA)
+
+# The whole JSON line stays under this many characters (a record that keeps
+# the last 8,000 characters of the output then holds all of it).
+LINE_LIMIT = 7500
+
+# Which yardstick (see measure_yardsticks) bounds which workload's whole call.
+YARDSTICK_OF = {
+    "c2_segreduce_f32": "read_nt_256MiB",
+    "c3_load_balance_search": "store_1GiB_runs_read2KB",
+    "c3_interval_expand_i32": "store_1GiB_runs_read2KB",
+}
+
+
+def sig(x, digits=5):
+    """x rounded to `digits` significant digits (None and ints pass through)."""
+    if x is None or isinstance(x, (int, str, bool)):
+        return x
+    return float("%.*g" % (digits, x))
+
+
+def compact(res, yardsticks):
+    """What the line keeps of a workload beside the headline."""
+    r = res["roofline"]
+    out = {"ms_per_step": sig(res["ms_per_step"]),
+           "median_ms_per_step": sig(res["median_ms_per_step"]),
+           "sustained_ms_per_step": sig(res["sustained_ms_per_step"]),
+           "pct_hbm_peak": sig(res["pct_hbm_peak"], 4),
+           "roofline": {"kernel": r["kernel"], "frac": sig(r["frac"], 4),
+                        "kernel_ms": sig(r["kernel_ms"]), "traffic": r["traffic"]}}
+    y = yardsticks.get(YARDSTICK_OF.get(res["workload"]))
+    if y:
+        out["frac_of_yardstick"] = sig(y / res["ms_per_step"], 4)
+    if "cpu_baseline" in res:
+        out["cpu_baseline"] = {"value": sig(res["cpu_baseline"]["value"], 4),
+                               "cores": res["cpu_baseline"]["cores"]}
+    return out
+
+
+def format_line(main_res, others, yardsticks, device, steps, warmup, copies):
+    """The one JSON line: the contract's keys for the headline workload, the
+    yardsticks, then the other workloads (compact, BASELINE's configs last)."""
+    roof = dict(main_res["roofline"])
+    for k in ("achieved", "frac", "kernel_ms"):
+        roof[k] = sig(roof[k])
+    line = {
+        "metric": "segreduce_input_GBps", "value": sig(main_res["GBps"]), "unit": "GB/s",
+        "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": sig(main_res["ms_per_step"]),
+        "median_ms_per_step": sig(main_res["median_ms_per_step"]),
+        "sustained_ms_per_step": sig(main_res["sustained_ms_per_step"]),
+        "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
+        "data": "synthetic (seeded numpy PCG64, seed 42), inputs resident in HBM, "
+                "%d rotating copies" % copies,
+        "config": {"workload": main_res["workload"], "description": main_res["description"],
+                   "algorithmic_bytes": main_res["algorithmic_bytes"]},
+        "items_per_s": sig(main_res["items_per_s"]),
+        "pct_hbm_peak": sig(main_res["pct_hbm_peak"], 4),
+        "roofline": roof,
+    }
+    y = yardsticks.get(YARDSTICK_OF.get(main_res["workload"]))
+    if y:
+        line["frac_of_yardstick"] = sig(y / main_res["ms_per_step"], 4)
+    if "cpu_baseline" in main_res:
+        c = dict(main_res["cpu_baseline"])
+        for k in ("value", "items_per_s", "single_thread_value"):
+            if k in c:
+                c[k] = sig(c[k], 4)
+        line["cpu_baseline"] = c
+    line["device"] = device
+    if yardsticks:
+        line["yardsticks"] = {"unit": "ms per launch; kernels that only read or only store "
+                                      "(tests/csrc/test_kernels.hip), not library kernels"}
+        line["yardsticks"].update({k: sig(v) for k, v in yardsticks.items()})
+    if others:
+        first = [k for k in others if k not in BASELINE_EXTRA]
+        last = [k for k in BASELINE_EXTRA if k in others]
+        line["others"] = {k: (others[k] if "error" in others[k] else
+                              compact(others[k], yardsticks)) for k in first + last}
+    return json.dumps(line, separators=(",", ":"))
+
+
+def measure_yardsticks(steps, warmup):
+    """Times of kernels that only read or only store, on this box, beside the
+    library's kernels (ms per launch, `steps` launches between two
+    synchronisations like a workload's steps):
+      read_nt_256MiB            bare non-temporal read of 256 MiB (what the
+                                2^26-float segreduce has to stream in),
+                                rotating over 4 buffers
+      store_1GiB_runs           1 GiB of ints stored as ragged tiles like the
+                                search's, runs of 16 tiles per XCD
+      store_1GiB_runs_read2KB   the same with 2 KB read per tile before it stores
+      store_1GiB_eighths        the same stores, one eighth of the tiles per XCD
+      read_64MiB_behind_store_1GiB   a 64 MiB read launched right behind that
+                                store kernel (event pair around the read alone):
+                                what a partition kernel over 2^24 starts meets
+                                when it follows a call that has just stored 1 GiB"""
+    import ctypes
+    import torch
+    tk = ctypes.CDLL(os.path.join(ROOT, "tests", "csrc", "libmgpu_test_kernels.so"))
+    tk.tk_read_probe.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int,
+                                 ctypes.c_void_p, ctypes.c_void_p]
+    stream = lambda: ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    res = {}
+    n = (256 << 20) // 4
+    bufs = [torch.randint(0, 1 << 30, (n,), dtype=torch.int32, device="cuda")
+            for _ in range(4)]
+
+    def read(i, nbytes=256 << 20):
+        rc = tk.tk_read_probe(bufs[i % 4].data_ptr(), nbytes, 1, None, stream())
+        assert rc == 0, rc
+    res["read_nt_256MiB"] = time_steps(read, steps, warmup) * 1e3
+
+    probes = {"store_1GiB_runs": make_store_probe(2, 1, 0),
+              "store_1GiB_runs_read2KB": make_store_probe(2, 1, 512),
+              "store_1GiB_eighths": make_store_probe(2, 2, 0)}
+    for key, wk in probes.items():
+        res[key] = time_steps(wk.step, steps, warmup) * 1e3
+
+    wk = probes["store_1GiB_runs"]
+    pairs = []
+    for i in range(warmup + max(steps, 10)):
+        wk.step(i)
+        e0 = torch.cuda.Event(enable_timing=True)
+        e1 = torch.cuda.Event(enable_timing=True)
+        e0.record()
+        read(i, 64 << 20)
+        e1.record()
+        if i >= warmup:
+            pairs.append((e0, e1))
+    torch.cuda.synchronize()
+    res["read_64MiB_behind_store_1GiB"] = sum(a.elapsed_time(b) for a, b in pairs) / len(pairs)
+    del probes, wk, bufs
+    torch.cuda.empty_cache()
+    return res
 
 
 def main():
@@ -927,6 +1065,7 @@ def main():
                     % ", ".join(sorted(FACTORIES)))
     ap.add_argument("--copies", type=int, default=4)
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-yardsticks", action="store_true")
     ap.add_argument("--extra", default=DEFAULT_EXTRA,
                     help="comma-separated further workloads reported under 'others'")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -989,7 +1128,6 @@ def main():
             "GBps": wk.bytes / sec / 1e9,
             "items_per_s": wk.items / sec,
             "pct_hbm_peak": 100.0 * wk.bytes / sec / 1e9 / HBM_PEAK_GBPS,
-            "pct_hbm_peak_median": 100.0 * wk.bytes / median / 1e9 / HBM_PEAK_GBPS,
             "algorithmic_bytes": wk.bytes,
             "roofline": {
                 "bound": "hbm", "kernel": wk.kernel,
@@ -1008,15 +1146,12 @@ def main():
     props = torch.cuda.get_device_properties(0)
     device = {"name": props.name, "compute_units": props.multi_processor_count,
               "hbm_peak_used_GBps": HBM_PEAK_GBPS,
-              # hipDeviceProp_t's memory clock and bus width, and clock x 2 x
-              # width / 8, the product mgpu's device_prop_string prints.  The
-              # runtime reports 2,000 MHz x 8,192 bits on MI355X, which that
-              # double-data-rate formula turns into 4,096 GB/s; HBM3E moves
-              # 8 Gb/s per pin (four bits per reported clock), so the fractions
-              # here are taken of the published 8 TB/s.
-              "memory_clock_khz": clock_khz.value, "memory_bus_width_bits": bus_bits.value,
-              "hbm_peak_from_device_properties_GBps":
-                  2.0 * clock_khz.value * 1e3 * bus_bits.value / 8 / 1e9}
+              # hipDeviceProp_t's memory clock and bus width.  The reference's
+              # device_prop_string prints clock x 2 x width / 8 = 4,096 GB/s
+              # for the 2,000 MHz x 8,192 bits the runtime reports; HBM3E
+              # moves 8 Gb/s per pin (four bits per reported clock), so the
+              # fractions here are taken of the published 8 TB/s.
+              "memory_clock_khz": clock_khz.value, "memory_bus_width_bits": bus_bits.value}
 
     main_res = measure(args.workload, True)
     others = {}
@@ -1024,40 +1159,19 @@ def main():
         # A further workload that fails (its parity check included) is
         # reported as failed; it does not take the headline with it.
         try:
-            r = measure(key, False)
+            others[key] = measure(key, False)
         except (Exception, SystemExit) as e:
-            others[key] = {"error": str(e) or type(e).__name__}
+            others[key] = {"error": (str(e) or type(e).__name__)[:120]}
             torch.cuda.empty_cache()
-            continue
-        others[key] = {k: r[k] for k in (
-            "description", "dtype", "ms_per_step", "median_ms_per_step",
-            "sustained_ms_per_step", "GBps", "items_per_s",
-            "pct_hbm_peak", "pct_hbm_peak_median", "algorithmic_bytes", "roofline")}
-        if "cpu_baseline" in r:
-            others[key]["cpu_baseline"] = r["cpu_baseline"]
-
-    line = {
-        "metric": "segreduce_input_GBps", "value": main_res["GBps"], "unit": "GB/s",
-        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
-        "ms_per_step": main_res["ms_per_step"],
-        "median_ms_per_step": main_res["median_ms_per_step"],
-        "sustained_ms_per_step": main_res["sustained_ms_per_step"],
-        "higher_is_better": True,
-        "scaling": "weak", "vs_baseline": None, "dtype": main_res["dtype"],
-        "data": "synthetic (seeded numpy PCG64, seed 42), inputs resident in HBM, "
-                "%d rotating copies" % args.copies,
-        "config": {"workload": main_res["workload"], "description": main_res["description"],
-                   "algorithmic_bytes": main_res["algorithmic_bytes"]},
-        "items_per_s": main_res["items_per_s"], "pct_hbm_peak": main_res["pct_hbm_peak"],
-        "pct_hbm_peak_median": main_res["pct_hbm_peak_median"],
-        "roofline": main_res["roofline"],
-    }
-    if "cpu_baseline" in main_res:
-        line["cpu_baseline"] = main_res["cpu_baseline"]
-    line["device"] = device
-    if others:
-        line["others"] = others
-    print(json.dumps(line))
+    yardsticks = {}
+    if not args.no_yardsticks:
+        try:
+            yardsticks = measure_yardsticks(args.steps, args.warmup)
+        except (Exception, SystemExit) as e:
+            yardsticks = {}
+            print("yardsticks failed: %s" % e, file=sys.stderr)
+    print(format_line(main_res, others, yardsticks, device, args.steps, args.warmup,
+                      args.copies))
 
 
 if __name__ == "__main__":

@@ -125,7 +125,13 @@ MGPU_HIP_API int mgpu_hip_segreduce(const void* input, int count,
  *  - All calls on one GPU share the one array: two calls may not overlap in
  *    time on the same GPU (different streams, or graphs replayed
  *    concurrently), they would race on it.  Calls on one stream are ordered
- *    and need nothing else. */
+ *    and need nothing else.
+ *  - The first call on each device looks the array's address up
+ *    (hipGetSymbolAddress: not a stream operation, and it may load the
+ *    library's code object, which allocates).  A caller that must not
+ *    allocate from some point on -- one that is about to capture a graph --
+ *    makes one call with count = 0 on that device before that point: it
+ *    enqueues nothing and resolves the address. */
 #define MGPU_HIP_STATIC_SCRATCH_BYTES (4u << 20)
 MGPU_HIP_API int mgpu_hip_segreduce_static(const void* input, int count,
   const int* segments, int num_segments, void* output, int dtype, int op,

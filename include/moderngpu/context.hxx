@@ -98,9 +98,11 @@ protected:
   // again may still be in use by kernels queued earlier on this context's
   // stream, so whoever gets it has to touch it through that stream only:
   // the library's kernels do, and so do to_mem(), from_mem() and
-  // mem_t::clone().  The raw-pointer copies htod()/dtoh()/dtod() run on the
-  // null stream, which a stream created with hipStreamNonBlocking does not
-  // wait for: call synchronize() first when the context has such a stream.
+  // mem_t::clone() and the htod()/dtoh()/dtod() overloads that take the
+  // context.  The raw-pointer copies without a context run on the null
+  // stream, which a stream created with hipStreamNonBlocking does not wait
+  // for: pass the context, or call synchronize() first, when the context has
+  // such a stream.
   std::multimap<size_t, void*> _free_blocks;
   std::unordered_map<void*, size_t> _live_blocks;
   size_t _cached_bytes;

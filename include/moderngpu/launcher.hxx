@@ -88,17 +88,14 @@ inline void launcher_check(int code) {
 }
 
 // Number of calls that went to the library (for tests).  With the environment
-// variable MGPU_HIP_LAUNCHER_REPORT set, the count is printed to stderr when
-// the program ends ("mgpu launcher calls: N"), and a line when the first call
-// is made (a program that is ended from outside never gets to the other):
-// that is how a program that cannot be edited -- one written for the CUDA
-// library and only recompiled -- shows which way its calls went.
+// variable MGPU_HIP_LAUNCHER_REPORT set, a program built with
+// MGPU_HIP_LAUNCHER prints the count to stderr when it ends ("mgpu launcher
+// calls: N", also when N is 0), and a line when the first call is made (a
+// program that is ended from outside never gets to the other): that is how a
+// program that cannot be edited -- one written for the CUDA library and only
+// recompiled -- shows which way its calls went.
 struct launcher_counter_t {
   long calls = 0;
-  launcher_counter_t() {
-    if(getenv("MGPU_HIP_LAUNCHER_REPORT"))
-      fprintf(stderr, "mgpu launcher: first call\n");
-  }
   ~launcher_counter_t() {
     if(getenv("MGPU_HIP_LAUNCHER_REPORT"))
       fprintf(stderr, "mgpu launcher calls: %ld\n", calls);
@@ -108,6 +105,16 @@ inline long& launcher_calls() {
   static launcher_counter_t counter;
   return counter.calls;
 }
+inline void launcher_count_call() {
+  long& calls = launcher_calls();
+  if(!calls++ && getenv("MGPU_HIP_LAUNCHER_REPORT"))
+    fprintf(stderr, "mgpu launcher: first call\n");
+}
+#ifdef MGPU_HIP_LAUNCHER
+// The counter exists from program start in a build with the dispatch layer,
+// so that its report at exit is printed whether or not a call went there.
+static long* const launcher_counter_from_start = &launcher_calls();
+#endif
 
 template<typename launch_arg_t, typename input_it, typename segments_it,
   typename output_it, typename op_t, typename type_t>
@@ -127,7 +134,7 @@ bool launcher_segreduce(input_it input, int count, segments_it segments,
     launcher_check(mgpu_hip_segreduce(input, count, segments, num_segments,
       output, dtype, launcher_op_t<op_t, type_t>::value, &init,
       workspace.data(), bytes, context.stream()));
-    ++launcher_calls();
+    launcher_count_call();
     return true;
   } else
     return false;
@@ -154,7 +161,7 @@ bool launcher_spmv(matrix_it matrix, columns_it columns, vector_it vector,
     launcher_check(mgpu_hip_spmv(matrix, columns, vector, count, segments,
       num_segments, output, dtype, workspace.data(), bytes,
       context.stream()));
-    ++launcher_calls();
+    launcher_count_call();
     return true;
   } else
     return false;
@@ -170,7 +177,7 @@ bool launcher_load_balance_search(int count, segments_it segments,
     mem_t<char> workspace(bytes, context);
     launcher_check(mgpu_hip_load_balance_search(count, segments,
       num_segments, output, workspace.data(), bytes, context.stream()));
-    ++launcher_calls();
+    launcher_count_call();
     return true;
   } else
     return false;
@@ -214,7 +221,7 @@ bool launcher_interval(input_it input, int count,
       code = mgpu_hip_interval_expand(input, size, count, segments,
         num_segments, output, ws, bytes, stream);
     launcher_check(code);
-    ++launcher_calls();
+    launcher_count_call();
     return true;
   } else
     return false;
@@ -245,7 +252,7 @@ bool launcher_scan(bool inclusive, input_it input, int count,
     launcher_check(mgpu_hip_scan(input, count, output, dtype,
       launcher_op_t<op_t, type_t>::value, (int)inclusive, total,
       workspace.data(), bytes, context.stream()));
-    ++launcher_calls();
+    launcher_count_call();
     return true;
   } else
     return false;
@@ -267,7 +274,7 @@ bool launcher_reduce(input_it input, int count, output_it reduction, op_t,
     launcher_check(mgpu_hip_reduce(input, count, reduction, dtype,
       launcher_op_t<op_t, type_t>::value, workspace.data(), bytes,
       context.stream()));
-    ++launcher_calls();
+    launcher_count_call();
     return true;
   } else
     return false;
@@ -290,7 +297,7 @@ bool launcher_sorted_search(bool upper, needles_it needles, int num_needles,
     launcher_check(mgpu_hip_sorted_search(needles, num_needles, haystack,
       num_haystack, upper ? MGPU_BOUNDS_UPPER : MGPU_BOUNDS_LOWER, indices,
       workspace.data(), bytes, context.stream()));
-    ++launcher_calls();
+    launcher_count_call();
     return true;
   } else
     return false;
@@ -318,7 +325,7 @@ bool launcher_inner_join(a_it a, int a_count, b_it b, int b_count, comp_t,
     launcher_check(mgpu_hip_inner_join_pairs(a_count, b_count, join_count,
       workspace.data(), (int*)output.data(), pairs_workspace.data(),
       pairs_bytes, context.stream()));
-    ++launcher_calls();
+    launcher_count_call();
     return true;
   } else
     return false;
@@ -331,7 +338,7 @@ bool launcher_load_balance_partitions(int64_t count, segments_it segments,
   if constexpr(launcher_points_to_t<segments_it, int>::value) {
     launcher_check(mgpu_hip_load_balance_partitions(count, segments,
       num_segments, spacing, partitions, context.stream()));
-    ++launcher_calls();
+    launcher_count_call();
     return true;
   } else
     return false;

@@ -84,6 +84,42 @@ hipError_t htod(type_t* dest, const std::vector<type_t>& source) {
   return htod(dest, source.data(), source.size());
 }
 
+// The same copies on a context's stream, waited for: the forms to use with
+// memory that came from that context when its stream does not synchronise with
+// the null stream (hipStreamNonBlocking) -- the block may be a recycled one
+// that kernels queued earlier on the stream still use, and only a copy on the
+// same stream is ordered behind them.  (No counterpart in the CUDA library,
+// whose contexts return blocks with a cudaFree that waits for the device.)
+template<typename type_t>
+hipError_t dtoh(type_t* dest, const type_t* source, size_t count,
+  context_t& context) {
+  return detail::copy_elements<hipMemcpyDeviceToHost>(dest, source, count,
+    context);
+}
+template<typename type_t>
+hipError_t htod(type_t* dest, const type_t* source, size_t count,
+  context_t& context) {
+  return detail::copy_elements<hipMemcpyHostToDevice>(dest, source, count,
+    context);
+}
+template<typename type_t>
+hipError_t dtod(type_t* dest, const type_t* source, size_t count,
+  context_t& context) {
+  return detail::copy_elements<hipMemcpyDeviceToDevice>(dest, source, count,
+    context);
+}
+template<typename type_t>
+hipError_t dtoh(std::vector<type_t>& dest, const type_t* source,
+  size_t count, context_t& context) {
+  dest.resize(count);
+  return dtoh(dest.data(), source, count, context);
+}
+template<typename type_t>
+hipError_t htod(type_t* dest, const std::vector<type_t>& source,
+  context_t& context) {
+  return htod(dest, source.data(), source.size(), context);
+}
+
 ////////////////////////////////////////////////////////////////////////////////
 // mem_t factories.
 

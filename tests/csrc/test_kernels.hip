@@ -351,3 +351,45 @@ API int tk_store_probe(int* out, const int* begins, int num_tiles,
   }
   return (int)hipGetLastError();
 }
+
+////////////////////////////////////////////////////////////////////////////////
+// A yardstick for the kernels that are streams of loads (segreduce, reduce):
+// CTAs of 256 threads read 16 KB each with 16-byte loads, non-temporal or
+// ordinary, and store nothing (a store guarded by a value the data never
+// folds to keeps the loads alive).  Launches on `stream` and does not wait.
+
+namespace {
+template<bool nontemporal>
+__global__ __launch_bounds__(256) void read_probe_k(const int* in,
+  size_t chunks, int* sink) {
+  typedef int v4_t __attribute__((ext_vector_type(4)));
+  const v4_t* p = (const v4_t*)in;
+  size_t base = (size_t)blockIdx.x * 1024 + threadIdx.x;
+  v4_t x[4];
+  PRAGMA_UNROLL
+  for(int i = 0; i < 4; ++i) {
+    size_t at = base + 256 * i;
+    if(at >= chunks) at = chunks - 1;
+    x[i] = nontemporal ? __builtin_nontemporal_load(p + at) : p[at];
+  }
+  int acc = 0;
+  PRAGMA_UNROLL
+  for(int i = 0; i < 4; ++i) acc ^= x[i].x ^ x[i].y ^ x[i].z ^ x[i].w;
+  if(0x5bd1e995 == acc && sink) sink[0] = acc;
+}
+} // namespace
+
+API int tk_read_probe(const int* in, size_t bytes, int nontemporal,
+  int* sink, void* stream) {
+  size_t chunks = bytes / 16;
+  if(!chunks || chunks > ((size_t)1 << 40)) return (int)hipErrorInvalidValue;
+  int grid = (int)((chunks + 1023) / 1024);
+  hipStream_t s = (hipStream_t)stream;
+  if(nontemporal)
+    hipLaunchKernelGGL(read_probe_k<true>, dim3(grid), dim3(256), 0, s, in,
+      chunks, sink);
+  else
+    hipLaunchKernelGGL(read_probe_k<false>, dim3(grid), dim3(256), 0, s, in,
+      chunks, sink);
+  return (int)hipGetLastError();
+}

@@ -142,6 +142,17 @@ static int check_memory(context_t& context) {
   CHECK(hipSuccess == htod(second.data(), elsewhere));
   CHECK(from_mem(second)[1] == 18);
 
+  // the same copies on the context's stream
+  mem_t<int64_t> third(count, context);
+  CHECK(hipSuccess == dtod(third.data(), counted.data(), count, context));
+  std::vector<int64_t> again;
+  CHECK(hipSuccess == dtoh(again, third.data() + 20, 3, context));
+  CHECK(again.size() == 3 && again[0] == 27 && again[2] == 29);
+  CHECK(hipSuccess == htod(third.data(), again, context));
+  CHECK(hipSuccess == htod(third.data() + 3, again.data(), 2, context));
+  std::vector<int64_t> t5 = from_mem(third);
+  CHECK(t5[0] == 27 && t5[2] == 29 && t5[3] == 27 && t5[4] == 28 && t5[5] == 12);
+
   // pinned host memory, move semantics
   mem_t<int> pinned(16, context, memory_space_host);
   CHECK(memory_space_host == pinned.space());

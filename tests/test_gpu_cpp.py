@@ -23,8 +23,11 @@ def _run(name, *args, report=False):
 
 
 def _launcher_calls(stderr):
+    """The count a program built with MGPU_HIP_LAUNCHER reports at exit (also
+    when it is 0); None when there is no report, i.e. the program was built
+    without the dispatch layer."""
     found = re.findall(r"mgpu launcher calls: (\d+)", stderr)
-    return int(found[-1]) if found else 0
+    return int(found[-1]) if found else None
 
 
 # The same callers built with MGPU_HIP_LAUNCHER: the public templates call the
@@ -44,6 +47,7 @@ def test_callers_through_the_dispatch_layer(dev, name, args, expected):
     out, err = _run("launcher_" + name, *args, report=True)
     assert "passed" in out
     calls = _launcher_calls(err)
+    assert calls is not None, "no report: not built with MGPU_HIP_LAUNCHER? " + err[-500:]
     print(name, "calls into libmgpu_hip.so:", calls)
     if expected == "some":
         assert calls > 0, err[-500:]

@@ -43,8 +43,11 @@ def _run(name, limit=110):
 
 
 def _launcher_calls(text):
+    """The count a launcher_* program reports at exit (also when it is 0);
+    None when there is no report (a program built without the dispatch layer,
+    or one that was ended from outside)."""
     found = re.findall(r"mgpu launcher calls: (\d+)", text)
-    return int(found[-1]) if found else 0
+    return int(found[-1]) if found else None
 
 
 def _run_for_a_while(name, seconds, enough=None):
@@ -127,7 +130,7 @@ def test_reference_test_reduce(dev, name):
     assert code == 0, out[-2000:] + err[-2000:]
     assert "ERROR" not in out
     assert out.count("success") > 1000
-    assert _launcher_calls(err) == 0
+    assert _launcher_calls(err) == (0 if name.startswith("launcher_") else None)
 
 
 @pytest.mark.parametrize("name", ["test_segreduce", "launcher_test_segreduce"])
@@ -154,14 +157,16 @@ def test_reference_test_merge(dev, name):
     # Sizes from 1,000 to 10^8 in steps of 10 %, each merged on the device and
     # with std::merge (the inputs are sorted on the host, which takes most of
     # the time at the large sizes); ended after a while like test_segreduce.
-    # Stops at 60 sizes or 60 s; passes with at least one size and no failure.
+    # Stops at 60 sizes or 60 s; passes with no failure among at least the
+    # first 25 sizes (1,000 to about 10,000 keys in all, a few milliseconds each on any
+    # host: from one tile of the merge kernel to several).
     # merge is not among the calls the C layer covers: in place either way.
     code, out = _run_for_a_while(name, 60,
                                  enough=lambda text: text.count("SUCCESS") >= 60)
     print(out[-400:])
     assert code in (None, 0), out[-2000:]
     assert "FAILURE" not in out
-    assert out.count("SUCCESS") >= 1, out[-2000:]
+    assert out.count("SUCCESS") >= 25, out[-2000:]
 
 
 @pytest.mark.parametrize("prefix", ["", "launcher_"])

@@ -77,3 +77,46 @@ def test_disk_cache_returns_the_same_arrays(tmp_path, monkeypatch):
     monkeypatch.delenv("MGPU_WORKLOAD_CACHE")
     plain = w.config5(scale=256, kind="i64sum")
     assert np.array_equal(plain["values"], first["values"])
+
+
+def test_bench_line_fits_the_record():
+    """The one JSON line of a default bench run, with every workload present
+    and every number at full width, stays under bench.LINE_LIMIT characters, so
+    that a record keeping the last 8,000 characters of the output holds the
+    whole line -- and BASELINE's configurations come last in it."""
+    import json
+    import os
+    import sys
+    sys.path.insert(0, os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+    import bench
+
+    def result(key):
+        return {"workload": key, "description": "d" * 90, "dtype": "f32",
+                "ms_per_step": 0.123456789, "median_ms_per_step": 0.123456789,
+                "sustained_ms_per_step": 0.123456789, "GBps": 5555.123456789,
+                "items_per_s": 1.23456789e12, "pct_hbm_peak": 69.123456789,
+                "algorithmic_bytes": 1207959552,
+                "roofline": {"bound": "hbm", "kernel": "k" * 56, "achieved": 5555.123456789,
+                             "peak": 8000.0, "unit": "GB/s", "frac": 0.70123456789,
+                             "kernel_ms": 0.123456789, "traffic": 1207959552},
+                "cpu_baseline": {"value": 11.123456789, "unit": "GB/s", "cores": 16,
+                                 "kind": "port", "items_per_s": 1.23456789e9,
+                                 "single_thread_value": 10.123456789, "sample": "s" * 160}}
+    keys = [k for k in bench.DEFAULT_EXTRA.split(",")]
+    assert set(bench.BASELINE_EXTRA) <= set(keys)
+    others = {k: result(k) for k in keys}
+    yard = {k: 0.123456789 for k in ("read_nt_256MiB", "store_1GiB_runs",
+                                     "store_1GiB_runs_read2KB", "store_1GiB_eighths",
+                                     "read_64MiB_behind_store_1GiB")}
+    device = {"name": "AMD Instinct MI355X", "compute_units": 256, "hbm_peak_used_GBps": 8000.0,
+              "memory_clock_khz": 2000000, "memory_bus_width_bits": 8192}
+    line = bench.format_line(result("c2_segreduce_f32"), others, yard, device, 20, 5, 4)
+    assert len(line) < bench.LINE_LIMIT, len(line)
+    parsed = json.loads(line)
+    for k in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+              "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config",
+              "roofline", "cpu_baseline"):
+        assert k in parsed
+    assert list(parsed["others"])[-len(bench.BASELINE_EXTRA):] == list(bench.BASELINE_EXTRA)
+    assert parsed["others"]["c3_load_balance_search"]["frac_of_yardstick"] == 1.0
+    assert bench.sig(0.123456789) == 0.12346 and bench.sig(7) == 7 and bench.sig(None) is None

@@ -48,6 +48,33 @@ def test_static_matches_workspace_entry_point_twice(dev, oracle):
     assert np.array_equal(got, want) and got[0] == vals.max()
 
 
+def test_static_call_allocates_no_device_memory(dev):
+    """After one empty call on the device (it resolves the address of the
+    library's array), a call through the C ABI leaves the device's free memory
+    as it was: nothing is allocated, by the library or by the runtime."""
+    L = m.lib()
+    w = workloads.config2(scale=64)                       # 2^20 floats, 2^14 segments
+    v = torch.from_numpy(w["values"]).to(dev)
+    s = torch.from_numpy(w["segments"]).to(dev)
+    out = torch.empty(s.numel(), dtype=torch.float32, device=dev)
+    init = ctypes.c_float(0.0)
+    stream = ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+    args = (ctypes.c_void_p(v.data_ptr()), v.numel(), ctypes.c_void_p(s.data_ptr()), s.numel(),
+            ctypes.c_void_p(out.data_ptr()), 4, 0, ctypes.byref(init), stream)   # MGPU_F32, plus
+    # The warm-up call: count = 0, nothing is enqueued.
+    assert L.mgpu_hip_segreduce_static(None, 0, None, 0, None, 4, 0, ctypes.byref(init),
+                                       stream) == 0
+    torch.cuda.synchronize()
+    free_before, _ = torch.cuda.mem_get_info()
+    for _ in range(3):
+        assert L.mgpu_hip_segreduce_static(*args) == 0
+    torch.cuda.synchronize()
+    free_after, _ = torch.cuda.mem_get_info()
+    assert free_after == free_before
+    want = m.segreduce(v, s, "plus", 0.0)
+    assert torch.equal(out, want)
+
+
 def test_static_rejects_what_does_not_fit(dev):
     L = m.lib()
     limit = 4 << 20
