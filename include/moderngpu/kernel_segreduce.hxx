@@ -275,6 +275,16 @@ struct segreduce_tile_f {
     flag_words = nv / 32 + 2
   };
   static_assert(vt <= 32, "segreduce tiles hold at most 32 values/thread");
+  enum {
+    // dense_tile() keeps the tile's starts in the part of the values' LDS
+    // that the items leave free, which they do for values of 4 bytes or more
+    // (a_count + b_count <= nv).
+    can_stage_starts = sizeof(type_t) >= sizeof(int),
+    // Rows of nt 16-byte loads that cover the b_count + 1 <= nv + 1 starts.
+    start_rows = (nv + 4 * nt) / (4 * nt),
+    // Longest run of items a single thread folds by itself there.
+    fold_max = 32
+  };
   typedef tile_layout_t<W> layout_t;
   typedef cta_segscan_t<nt, type_t> segscan_t;
   typedef tile_loader_t<input_it, type_t, W> loader_t;
@@ -326,6 +336,14 @@ struct segreduce_tile_f {
     // load or LDS store needs a per-lane bounds check.  The kernel body
     // exists once for such tiles and once with the checks.
     // Computed items exist for the tile's own index range only.
+    // A tile with more segment starts than threads goes another way
+    // (dense_tile).
+    if constexpr(can_stage_starts) {
+      if(range.b_count() > nt) {
+        dense_tile(tid, cta, range, shared, args...);
+        return;
+      }
+    }
     if(!is_lbs_input_t<input_it>::value && range.a_begin <= count - nv)
       tile(std::true_type(), tid, cta, range, shared, args...);
     else
@@ -370,6 +388,95 @@ struct segreduce_tile_f {
       }
       // The search's LDS is about to hold the values.
       __syncthreads();
+    }
+  }
+
+  // Steps 3 to 5 of the tile: the items are in LDS (padded layout) and the
+  // start bits in shared.flags; afterwards LDS slot e holds the fold of its
+  // segment from max(segment start, start of e's thread) to e, and
+  // shared.flow[t] the fold that flows into thread t.  Ends with a barrier.
+  template<typename interior_t>
+  MGPU_DEVICE void scan_items(interior_t, int tid, int a_count,
+    work_storage_t& shared) const {
+    enum { interior = interior_t::value };
+    // Thread order: items [vt * tid, vt * tid + vt) and their start bits.
+    type_t x[vt];
+    PRAGMA_UNROLL
+    for(int c = 0; c < chunks; ++c) {
+      type_t chunk[W];
+      lds_load_chunk<W>(shared.values + layout_t::index(vt * tid + W * c),
+        chunk);
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) x[W * c + e] = chunk[e];
+    }
+    unsigned bits;
+    {
+      int pos = vt * tid;
+      unsigned long long two = shared.flags[pos >> 5] |
+        ((unsigned long long)shared.flags[(pos >> 5) + 1] << 32);
+      bits = (unsigned)(two >> (pos & 31));
+      if(vt < 32) bits &= (1u << vt) - 1;
+    }
+
+    // Inclusive segmented scan of the thread's items, left to right.
+    segscan_thread_t<1, vt>::run(x, ~bits, op);
+
+    PRAGMA_UNROLL
+    for(int c = 0; c < chunks; ++c) {
+      type_t chunk[W];
+      PRAGMA_UNROLL
+      for(int e = 0; e < W; ++e) chunk[e] = x[W * c + e];
+      if(interior || vt * tid + W * c < a_count)
+        lds_store_chunk<W>(shared.values + layout_t::index(vt * tid + W * c),
+          chunk);
+    }
+
+    segscan_result_t<type_t> flow = segscan_t().segscan(tid, 0 != bits, true,
+      x[vt - 1], shared.segscan, init, op);
+    shared.flow[tid] = flow.scan;
+    __syncthreads();
+
+  }
+
+  // Fold of tile items [p .. e] after scan_items(), where no segment starts
+  // inside (p, e].
+  MGPU_DEVICE type_t fold_to(const work_storage_t& shared, int p, int e) const {
+    int te = e / vt;
+    type_t v = shared.values[layout_t::index(e)];
+    // thread 0 has nothing flowing in; p may be negative for the segment
+    // that was open when the tile began.
+    if(te && p < te * vt) v = op(shared.flow[te], v);
+    return v;
+  }
+
+  // Fold of the tile's items [p, e), e > p, as they were loaded (before any
+  // scan), left to right by one thread.  (Reading two or four items ahead
+  // made tiles of 3- and 8-item segments 5 to 15 % slower.)
+  MGPU_DEVICE type_t fold_items(const work_storage_t& shared, int p,
+    int e) const {
+    type_t v = shared.values[layout_t::index(p)];
+    for(int q = p + 1; q < e; ++q)
+      v = op(v, shared.values[layout_t::index(q)]);
+    return v;
+  }
+
+  // The segment that was open when the tile began owns items [0, f), whose
+  // fold is `partial`.  Its code tells the spine which segment to fold the
+  // partial into, and whether that segment already has a value in output[]:
+  // it does unless its start was the very last merged element of its own tile
+  // (then that tile held none of its items and wrote nothing).  open_start is
+  // the start of that segment.  Called by one thread.
+  MGPU_DEVICE void emit_carry(int cta, merge_range_t range, int f,
+    int open_start, type_t partial) const {
+    if(f > 0 && range.b_begin > 0) {
+      int seg = range.b_begin - 1;
+      int node = open_start + seg;              // merged position of start
+      bool fresh = 0 == (node + 1) % nv;
+      carry_values[cta] = partial;
+      carry_codes[cta] = carry_code_t::make(seg, fresh);
+    } else {
+      carry_values[cta] = init;
+      carry_codes[cta] = carry_code_t::none;
     }
   }
 
@@ -435,52 +542,7 @@ struct segreduce_tile_f {
     }
     __syncthreads();
 
-    // Thread order: items [vt * tid, vt * tid + vt) and their start bits.
-    type_t x[vt];
-    PRAGMA_UNROLL
-    for(int c = 0; c < chunks; ++c) {
-      type_t chunk[W];
-      lds_load_chunk<W>(shared.values + layout_t::index(vt * tid + W * c),
-        chunk);
-      PRAGMA_UNROLL
-      for(int e = 0; e < W; ++e) x[W * c + e] = chunk[e];
-    }
-    unsigned bits;
-    {
-      int pos = vt * tid;
-      unsigned long long two = shared.flags[pos >> 5] |
-        ((unsigned long long)shared.flags[(pos >> 5) + 1] << 32);
-      bits = (unsigned)(two >> (pos & 31));
-      if(vt < 32) bits &= (1u << vt) - 1;
-    }
-
-    // Inclusive segmented scan of the thread's items, left to right.
-    segscan_thread_t<1, vt>::run(x, ~bits, op);
-
-    PRAGMA_UNROLL
-    for(int c = 0; c < chunks; ++c) {
-      type_t chunk[W];
-      PRAGMA_UNROLL
-      for(int e = 0; e < W; ++e) chunk[e] = x[W * c + e];
-      if(interior || vt * tid + W * c < a_count)
-        lds_store_chunk<W>(shared.values + layout_t::index(vt * tid + W * c),
-          chunk);
-    }
-
-    segscan_result_t<type_t> flow = segscan_t().segscan(tid, 0 != bits, true,
-      x[vt - 1], shared.segscan, init, op);
-    shared.flow[tid] = flow.scan;
-    __syncthreads();
-
-    // Fold of tile items [p .. e], where no segment starts inside (p, e].
-    auto fold_to = [&](int p, int e) -> type_t {
-      int te = e / vt;
-      type_t v = shared.values[layout_t::index(e)];
-      // thread 0 has nothing flowing in; p may be negative for the segment
-      // that was open when the tile began.
-      if(te && p < te * vt) v = op(shared.flow[te], v);
-      return v;
-    };
+    scan_items(interior_t(), tid, a_count, shared);
 
     // One thread per segment start of the tile.
     for(int j = tid; j < b_count; j += nt) {
@@ -494,31 +556,137 @@ struct segreduce_tile_f {
       if(next <= s) output[seg] = init;                  // empty segment
       else if(p >= 0 && p < a_count) {
         int e = min(next, range.a_end) - range.a_begin - 1;
-        output[seg] = fold_to(p, e);
+        output[seg] = fold_to(shared, p, e);
       }
       // else: the segment's first item is in the next tile; the spine
       // writes it.
     }
 
-    // The segment that was open when the tile began owns items [0, f).  Its
-    // code tells the spine which segment to fold the partial into, and
-    // whether that segment already has a value in output[]: it does unless
-    // its start was the very last merged element of its own tile (then that
-    // tile held none of its items and wrote nothing).
     if(!tid) {
       int f = a_count;
       if(b_count) f = min(max(first_start - range.a_begin, 0), a_count);
-      if(f > 0 && range.b_begin > 0) {
-        int seg = range.b_begin - 1;
-        int node = open_start + seg;              // merged position of start
-        bool fresh = 0 == (node + 1) % nv;
-        carry_values[cta] = fold_to(-1, f - 1);
-        carry_codes[cta] = carry_code_t::make(seg, fresh);
-      } else {
-        carry_values[cta] = init;
-        carry_codes[cta] = carry_code_t::none;
+      emit_carry(cta, range, f, open_start,
+        f > 0 ? fold_to(shared, -1, f - 1) : init);
+    }
+  }
+
+  // A tile with more segment starts than threads (segments of fewer than
+  // vt items on average).  What the ordinary path does per start -- an LDS
+  // atomic for its bit, a read of the start and of the one after it from
+  // global memory by whichever thread gets to write the segment's result --
+  // is most of the work of such a tile, so here the starts are read once,
+  // with 16-byte loads issued up front, and kept in LDS: in the part of the
+  // values' array that the items leave free (a_count + b_count <= nv).  If no
+  // segment has more than fold_max items inside the tile, the flag bits, the
+  // segmented scan and the CTA scan are left out altogether: one thread per
+  // start folds its segment's items straight from LDS, left to right, and
+  // stores the result.  Otherwise the tile continues as the ordinary path
+  // does, with its starts coming from LDS.
+  template<typename... args_t>
+  MGPU_DEVICE void dense_tile(int tid, int cta, merge_range_t range,
+    storage_t& storage, args_t... args) const {
+    work_storage_t& shared = storage.work;
+    int a_count = range.a_count();
+    int b_count = range.b_count();
+    // st[j] = start of segment b_begin + j for j in [0, b_count]; the start
+    // "after the last segment" is count.
+    int* st = (int*)(shared.values + layout_t::capacity(nv)) - (b_count + 1);
+    int open_start = 0;
+    if(!tid && range.b_begin > 0) open_start = segments[range.b_begin - 1];
+
+    // Computed items need the LDS for themselves first.
+    type_t r[chunks][W];
+    if constexpr(is_lbs_input_t<input_it>::value)
+      compute_items(range, tid, r, storage, args...);
+
+    int fetched[start_rows][4];
+    int available = min(b_count + 1, num_segments - range.b_begin);
+    PRAGMA_UNROLL
+    for(int row = 0; row < start_rows; ++row) {
+      int j = 4 * (nt * row + tid);
+      if(j < available)
+        cta_load_balance_t<nt, vt>::load_starts(segments, range.b_begin + j,
+          range.b_begin + available, fetched[row]);
+    }
+    if constexpr(!is_lbs_input_t<input_it>::value) {
+      PRAGMA_UNROLL
+      for(int i = 0; i < chunks; ++i) {
+        int p = W * (nt * i + tid);
+        if(p + W <= a_count)
+          loader_t::load(input, range.a_begin, (unsigned)p, r[i]);
+        else {
+          PRAGMA_UNROLL
+          for(int e = 0; e < W; ++e)
+            if(p + e < a_count) r[i][e] = input[range.a_begin + p + e];
+        }
       }
     }
+    for(int w = tid; w < flag_words; w += nt) shared.flags[w] = 0;
+    PRAGMA_UNROLL
+    for(int row = 0; row < start_rows; ++row) {
+      int j = 4 * (nt * row + tid);
+      PRAGMA_UNROLL
+      for(int e = 0; e < 4; ++e)
+        if(j + e <= b_count)
+          st[j + e] = (j + e < available) ? fetched[row][e] : count;
+    }
+    PRAGMA_UNROLL
+    for(int i = 0; i < chunks; ++i) {
+      int p = W * (nt * i + tid);
+      if(p < a_count)
+        lds_store_chunk<W>(shared.values + layout_t::index(p), r[i]);
+    }
+    __syncthreads();
+
+    // Items [0, f) belong to the segment that was open when the tile began.
+    int f = min(max(st[0] - range.a_begin, 0), a_count);
+    // The item ranges the starts own inside the tile: [p, e) for start j,
+    // empty for an empty segment.  (The clamps only matter for malformed
+    // input.)
+    auto owned = [&](int j, int& p, int& e) {
+      int s = st[j], next = st[j + 1];
+      p = min(max(s - range.a_begin, 0), a_count);
+      e = min(max(next - range.a_begin, p), a_count);
+      return next > s;
+    };
+    bool longer = !tid && f > fold_max;
+    for(int j = tid; j < b_count; j += nt) {
+      int p, e;
+      owned(j, p, e);
+      longer |= e - p > fold_max;
+    }
+
+    if(!__syncthreads_or(longer)) {
+      for(int j = tid; j < b_count; j += nt) {
+        int p, e;
+        bool filled = owned(j, p, e);
+        if(!filled) output[range.b_begin + j] = init;
+        else if(e > p) output[range.b_begin + j] = fold_items(shared, p, e);
+        // else: the segment's first item is in the next tile; the spine
+        // writes it.
+      }
+      if(!tid)
+        emit_carry(cta, range, f, open_start,
+          f > 0 ? fold_items(shared, 0, f) : init);
+      return;
+    }
+
+    // Some segment is long: bits, scan and flow as in the ordinary path.
+    for(int j = tid; j < b_count; j += nt) {
+      int p = min(max(st[j] - range.a_begin, 0), a_count);
+      atomicOr(&shared.flags[p >> 5], 1u << (p & 31));
+    }
+    __syncthreads();
+    scan_items(std::false_type(), tid, a_count, shared);
+    for(int j = tid; j < b_count; j += nt) {
+      int p, e;
+      bool filled = owned(j, p, e);
+      if(!filled) output[range.b_begin + j] = init;
+      else if(e > p) output[range.b_begin + j] = fold_to(shared, p, e - 1);
+    }
+    if(!tid)
+      emit_carry(cta, range, f, open_start,
+        f > 0 ? fold_to(shared, -1, f - 1) : init);
   }
 };
 

@@ -338,8 +338,16 @@ struct lbs_partition_search_f {
   }
 };
 
+// It is also used from 2^24 segments on, whatever the number of splits: the
+// scatter kernel reads every start (2^26 of them: 65 us, 22 M: 17 us), the
+// searches read 26 starts per split, the first dozen of which stay in the L2
+// (21 and 12 us; at 2^24 starts the two take the same time).
+#ifndef MGPU_LBS_SEARCH_FROM_SEGMENTS
+#define MGPU_LBS_SEARCH_FROM_SEGMENTS (1 << 24)
+#endif
 inline bool lbs_partition_by_search(int num_segments, int num_partitions) {
-  return (int64_t)num_partitions >= 2 * (int64_t)num_segments;
+  return (int64_t)num_partitions >= 2 * (int64_t)num_segments ||
+    num_segments >= MGPU_LBS_SEARCH_FROM_SEGMENTS;
 }
 
 // Copies of the scatter kernel's CTAs (see lbs_partition_scatter_f): one,

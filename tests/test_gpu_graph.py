@@ -65,3 +65,49 @@ def test_calls_recorded_in_a_graph_replay_correctly(oracle, dev):
         # eager work of the program between replays
         eager = m.segreduce(values, segments, "maximum", 0)
         assert np.array_equal(eager.cpu().numpy(), oracle.segreduce(v, segs, "maximum", 0))
+
+
+def test_large_call_recorded_in_a_graph_takes_new_segments(oracle, dev):
+    """A call of more than 4,096 tiles has a partition kernel in front of its
+    tile kernel (smaller ones let the tiles search their own splits).  The
+    replays here get new segment starts in the same buffer each time: the
+    partition has to run again in every replay, splits left by an earlier one
+    would give wrong sums."""
+    import moderngpu_amd as m
+    rng = np.random.default_rng(22)
+    nv = m.segreduce_tile_size(0)
+    count, nseg = 4200 * nv, 150_000
+    values = torch.zeros(count, dtype=torch.int32, device=dev)
+    segments = torch.zeros(nseg, dtype=torch.int32, device=dev)
+    reduced = torch.empty(nseg, dtype=torch.int32, device=dev)
+    owners = torch.empty(count, dtype=torch.int32, device=dev)
+
+    def calls():
+        m.segreduce(values, segments, "plus", -1, out=reduced)
+        m.load_balance_search(count, segments, out=owners)
+
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        calls()
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=side):
+        calls()
+
+    for replay in range(3):
+        v = rng.integers(-1000, 1000, count).astype(np.int32)
+        segs = np.sort(rng.integers(0, count, nseg)).astype(np.int32)
+        segs[0] = 0
+        values.copy_(torch.from_numpy(v).to(dev))
+        segments.copy_(torch.from_numpy(segs).to(dev))
+        reduced.fill_(-7)
+        owners.fill_(-7)
+        graph.replay()
+        torch.cuda.synchronize()
+        assert np.array_equal(reduced.cpu().numpy(), oracle.segreduce(v, segs, "plus", -1)), replay
+        assert np.array_equal(owners.cpu().numpy(), oracle.load_balance_search(count, segs)), replay
+        # the same call run eagerly between the replays
+        eager = m.segreduce(values, segments, "plus", -1)
+        assert torch.equal(eager, reduced), replay

@@ -120,6 +120,28 @@ def test_layouts_all_types(dev, oracle, dtype, op):
         _check(values, segs, op, init, oracle, name + "/partitioned", phases=7 | 8)
 
 
+@pytest.mark.parametrize("dtype", [np.int32, np.uint32, np.int64, np.uint64,
+                                   np.float32, np.float64])
+def test_short_segments_2p22(dev, oracle, dtype):
+    """2^22 items in segments of 1, 3 and 8 items (tiles with more starts than
+    threads, a thousand or more of them) and of 0 to 40 items at random, for
+    every value type: plus and maximum against the CPU loop."""
+    rng = np.random.default_rng(24)
+    count = 1 << 22
+    if np.dtype(dtype).kind == "f":
+        values = (rng.standard_normal(count) * 100).astype(dtype)
+    else:
+        info = np.iinfo(dtype)
+        values = rng.integers(info.min, info.max, size=count, dtype=dtype, endpoint=True)
+    layouts = [("len%d" % k, np.arange(0, count, k, dtype=np.int32)) for k in (1, 3, 8)]
+    lens = rng.integers(0, 41, size=count // 16)
+    starts = np.concatenate([[0], np.cumsum(lens)[:-1]])
+    layouts.append(("mixed", starts[starts <= count].astype(np.int32)))
+    for name, segs in layouts:
+        _check(values, segs, "plus", 3, oracle, name)
+        _check(values, segs, "maximum", 3, oracle, name)
+
+
 def test_float_specials(dev, oracle):
     # +0/-0 ties and infinities through max/min must match the host loop's
     # left-operand-wins rule bit for bit.

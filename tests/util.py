@@ -48,6 +48,21 @@ def segment_layouts(rng, nv):
     lens[[500, 1500, 2500, 3500]] = [3 * nv + 1, 7 * nv, nv, 2 * nv - 1]
     starts = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
     cases.append(("giants_among_units", int(lens.sum()), starts))
+    # tiles with more starts than threads: short segments of one length, of
+    # mixed lengths below and around the 32 items a thread folds by itself,
+    # and short ones with a long one in the middle of a tile
+    for length in (3, 8):
+        n = 3 * nv + 5
+        cases.append(("dense_len%d" % length, n, np.arange(0, n, length, dtype=np.int32)))
+    for top in (12, 33, 70):
+        lens = rng.integers(0, top + 1, size=nv)
+        starts = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+        cases.append(("dense_mixed_to_%d" % top, int(lens.sum()), starts))
+    lens = rng.integers(0, 4, size=2 * nv)
+    lens[nv // 3] = nv // 2 + 3
+    lens[nv] = 33
+    starts = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+    cases.append(("dense_with_long", int(lens.sum()), starts))
     for i in range(4):
         count = int(rng.integers(1, 6 * nv))
         nseg = int(rng.integers(1, 2 * nv))
