@@ -927,7 +927,7 @@ LINE_LIMIT = 7500
 YARDSTICK_OF = {
     "c2_segreduce_f32": "read_nt_256MiB",
     "c3_load_balance_search": "store_1GiB_runs_read2KB",
-    "c3_interval_expand_i32": "store_1GiB_runs_read2KB",
+    "c3_interval_expand_i32": "store_1GiB_runs_read4KB",
 }
 
 
@@ -1010,6 +1010,9 @@ def measure_yardsticks(steps, warmup):
       store_1GiB_runs           1 GiB of ints stored as ragged tiles like the
                                 search's, runs of 16 tiles per XCD
       store_1GiB_runs_read2KB   the same with 2 KB read per tile before it stores
+                                (the search reads about that much per tile)
+      store_1GiB_runs_read4KB   with 4 KB per tile (interval_expand: starts and
+                                values)
       store_1GiB_eighths        the same stores, one eighth of the tiles per XCD
       read_64MiB_behind_store_1GiB   a 64 MiB read launched right behind that
                                 store kernel (event pair around the read alone):
@@ -1033,6 +1036,7 @@ def measure_yardsticks(steps, warmup):
 
     probes = {"store_1GiB_runs": make_store_probe(2, 1, 0),
               "store_1GiB_runs_read2KB": make_store_probe(2, 1, 512),
+              "store_1GiB_runs_read4KB": make_store_probe(2, 1, 1024),
               "store_1GiB_eighths": make_store_probe(2, 2, 0)}
     for key, wk in probes.items():
         res[key] = time_steps(wk.step, steps, warmup) * 1e3

@@ -302,7 +302,7 @@ API int tk_load_balance(int nt, int vt, int count, const int* segments,
 // A yardstick for the kernels that are streams of stores (the load-balancing
 // search family): CTA `tile` stores the ints [begins[tile], begins[tile + 1])
 // with 16-byte stores, after reading read_ints ints of `source` (from
-// read_ints * tile on; read_ints <= 512) that the stored values depend on.
+// read_ints * tile on; read_ints <= 1024) that the stored values depend on.
 // mapping: 0 tile = blockIdx, 1 runs of 16 tiles per XCD (xcd_tile),
 // 2 one contiguous eighth of the tiles per XCD (xcd_tile_eighths).
 // The grid is xcd_grid(num_tiles).  Launches on `stream` and does not wait.
@@ -318,6 +318,7 @@ __global__ __launch_bounds__(512) void store_probe_k(int* out,
   __shared__ int exchange[512];
   int tid = threadIdx.x;
   int x = tid < read_ints ? source[(size_t)read_ints * tile + tid] : 0;
+  if(512 + tid < read_ints) x ^= source[(size_t)read_ints * tile + 512 + tid];
   exchange[tid] = x;
   __syncthreads();
   x = exchange[(tid + 1) % 512];
@@ -336,7 +337,7 @@ __global__ __launch_bounds__(512) void store_probe_k(int* out,
 
 API int tk_store_probe(int* out, const int* begins, int num_tiles,
   int mapping, int read_ints, const int* source, void* stream) {
-  if(num_tiles <= 0 || read_ints < 0 || read_ints > 512 ||
+  if(num_tiles <= 0 || read_ints < 0 || read_ints > 1024 ||
     mapping < 0 || mapping > 2)
     return (int)hipErrorInvalidValue;
   int grid = detail::xcd_grid(num_tiles);

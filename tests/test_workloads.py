@@ -106,7 +106,8 @@ def test_bench_line_fits_the_record():
     assert set(bench.BASELINE_EXTRA) <= set(keys)
     others = {k: result(k) for k in keys}
     yard = {k: 0.123456789 for k in ("read_nt_256MiB", "store_1GiB_runs",
-                                     "store_1GiB_runs_read2KB", "store_1GiB_eighths",
+                                     "store_1GiB_runs_read2KB", "store_1GiB_runs_read4KB",
+                                     "store_1GiB_eighths",
                                      "read_64MiB_behind_store_1GiB")}
     device = {"name": "AMD Instinct MI355X", "compute_units": 256, "hbm_peak_used_GBps": 8000.0,
               "memory_clock_khz": 2000000, "memory_bus_width_bits": 8192}
