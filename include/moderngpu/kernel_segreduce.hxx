@@ -278,8 +278,9 @@ struct segreduce_tile_f {
   enum {
     // dense_tile() keeps the tile's starts in the part of the values' LDS
     // that the items leave free, which they do for values of 4 bytes or more
-    // (a_count + b_count <= nv).
-    can_stage_starts = sizeof(type_t) >= sizeof(int),
+    // (a_count + b_count <= nv) that are aligned like an int.
+    can_stage_starts = sizeof(type_t) >= sizeof(int) &&
+      0 == alignof(type_t) % alignof(int),
     // Rows of nt 16-byte loads that cover the b_count + 1 <= nv + 1 starts.
     start_rows = (nv + 4 * nt) / (4 * nt),
     // Longest run of items a single thread folds by itself there.
