@@ -149,3 +149,48 @@ def test_large_random_shapes(oracle, dev):
         got = m.segreduce(torch.from_numpy(vals).to(dev), segs, "plus", -5)
         assert np.array_equal(got.cpu().numpy(),
                               oracle.segreduce(vals, starts, "plus", -5)), ("segreduce",) + tag
+
+
+@pytest.mark.parametrize("seed", range(24))
+def test_short_segments_fuzz(oracle, dev, seed):
+    """Inputs whose tiles hold more segment starts than threads: segments of a
+    few items, of lengths around the 32 items up to which a thread folds a
+    segment by itself, and short ones with a long one here and there (those
+    tiles fall back to the scan).  A few tiles each, with and without the
+    partition kernel; integer types, bit for bit."""
+    import moderngpu_amd as m
+    rng = np.random.default_rng(7000 + seed)
+    for _ in range(5):
+        nseg = int(rng.integers(300, 30_000))
+        kind = int(rng.integers(0, 4))
+        if kind == 0:
+            lens = np.full(nseg, int(rng.integers(1, 13)))
+        elif kind == 1:
+            lens = rng.integers(0, int(rng.choice([2, 4, 31, 32, 33, 34, 48])) + 1, size=nseg)
+        elif kind == 2:
+            lens = (rng.random(nseg) < 0.6).astype(np.int64)
+            where = rng.integers(0, nseg, size=int(rng.integers(1, 6)))
+            lens[where] = rng.integers(33, 9000, size=where.size)
+        else:
+            lens = rng.integers(0, 3, size=nseg)
+            lens[rng.integers(0, nseg, size=nseg // 50 + 1)] = 32
+            lens[rng.integers(0, nseg, size=3)] = 33
+        starts = np.concatenate([[0], np.cumsum(lens)[:-1]]).astype(np.int32)
+        count = int(lens.sum()) + int(rng.integers(0, 2)) * int(rng.integers(0, 100))
+        tag = (seed, kind, count, nseg)
+        segs = torch.from_numpy(starts).to(dev)
+        dtype = [np.int32, np.int64, np.uint32][int(rng.integers(0, 3))]
+        op = ["plus", "maximum", "minimum"][int(rng.integers(0, 3))]
+        values = rng.integers(0, 2000, size=count).astype(dtype)
+        want = oracle.segreduce(values, starts, op, 5)
+        dev_values = torch.from_numpy(values.view(np.int32) if dtype == np.uint32
+                                      else values).to(dev)
+        for phases in (7, 7 | 8):
+            got = m.segreduce(dev_values, segs, op, 5, unsigned=dtype == np.uint32,
+                              phases=phases).cpu().numpy()
+            got = got.view(np.uint32) if dtype == np.uint32 else got
+            assert np.array_equal(got, want), ("segreduce", phases, np.dtype(dtype).name, op) + tag
+        got = m.lbs_segreduce_seg_plus_rank(count, segs, init=-1)
+        assert np.array_equal(got.cpu().numpy(),
+                              oracle.lbs_segreduce_seg_plus_rank(count, starts, init=-1)), \
+            ("lbs_segreduce",) + tag
