@@ -284,7 +284,14 @@ struct segreduce_tile_f {
     // Rows of nt 16-byte loads that cover the b_count + 1 <= nv + 1 starts.
     start_rows = (nv + 4 * nt) / (4 * nt),
     // Longest run of items a single thread folds by itself there.
-    fold_max = 32
+    fold_max = 32,
+    // Starts (and the start after each) that a thread of an ordinary tile
+    // reads ahead into registers; tiles with more than start_regs * nt starts
+    // go to dense_tile().
+#ifndef MGPU_SEGREDUCE_START_REGS
+#define MGPU_SEGREDUCE_START_REGS 2
+#endif
+    start_regs = MGPU_SEGREDUCE_START_REGS
   };
   typedef tile_layout_t<W> layout_t;
   typedef cta_segscan_t<nt, type_t> segscan_t;
@@ -340,7 +347,7 @@ struct segreduce_tile_f {
     // A tile with more segment starts than threads goes another way
     // (dense_tile).
     if constexpr(can_stage_starts) {
-      if(range.b_count() > nt) {
+      if(range.b_count() > start_regs * nt) {
         dense_tile(tid, cta, range, shared, args...);
         return;
       }
@@ -500,6 +507,20 @@ struct segreduce_tile_f {
       first_start = segments[seg];
       first_next = (seg + 1 < num_segments) ? (int)segments[seg + 1] : count;
     }
+    // ... and the same for further starts of the thread, nt apart (tiles of
+    // up to start_regs * nt starts come this way).
+    int more_start[start_regs - 1 > 0 ? start_regs - 1 : 1];
+    int more_next[start_regs - 1 > 0 ? start_regs - 1 : 1];
+    PRAGMA_UNROLL
+    for(int k = 1; k < start_regs; ++k) {
+      more_start[k - 1] = more_next[k - 1] = 0;
+      if(nt * k + tid < b_count) {
+        int seg = range.b_begin + nt * k + tid;
+        more_start[k - 1] = segments[seg];
+        more_next[k - 1] = (seg + 1 < num_segments) ? (int)segments[seg + 1] :
+          count;
+      }
+    }
     if(!tid && range.b_begin > 0) open_start = segments[range.b_begin - 1];
     // The item loads; they are consumed after the flag setup.
     type_t r[chunks][W];
@@ -530,7 +551,16 @@ struct segreduce_tile_f {
     // One bit per segment start.  Starts of this tile lie in
     // [a_begin, a_end]; the clamp only guards against malformed input.
     for(int j = tid; j < b_count; j += nt) {
-      int s = (j == tid) ? first_start : (int)segments[range.b_begin + j];
+      int s = first_start;
+      if(j != tid) {
+        int k = (j - tid) / nt;
+        s = 0;
+        bool held = false;
+        PRAGMA_UNROLL
+        for(int q = 1; q < start_regs; ++q)
+          if(q == k) { s = more_start[q - 1]; held = true; }
+        if(!held) s = (int)segments[range.b_begin + j];
+      }
       int p = min(max(s - range.a_begin, 0), a_count);
       atomicOr(&shared.flags[p >> 5], 1u << (p & 31));
     }
@@ -550,8 +580,15 @@ struct segreduce_tile_f {
       int seg = range.b_begin + j;
       int s = first_start, next = first_next;
       if(j != tid) {
-        s = segments[seg];
-        next = (seg + 1 < num_segments) ? (int)segments[seg + 1] : count;
+        int k = (j - tid) / nt;
+        bool held = false;
+        PRAGMA_UNROLL
+        for(int q = 1; q < start_regs; ++q)
+          if(q == k) { s = more_start[q - 1]; next = more_next[q - 1]; held = true; }
+        if(!held) {
+          s = segments[seg];
+          next = (seg + 1 < num_segments) ? (int)segments[seg + 1] : count;
+        }
       }
       int p = s - range.a_begin;
       if(next <= s) output[seg] = init;                  // empty segment
