@@ -788,10 +788,16 @@ struct cta_load_balance_t {
         if(4 * q < loaded) stage(q, info.starts[r]);
       }
     } else {
-      for(int q = tid; 4 * q < loaded; q += nt) {
-        int x[4] = { 0, 0, 0, 0 };
-        load_starts(segments, jb + 4 * q, je, x);
-        stage(q, x);
+      // A tile of many starts: three rows of loads in flight at a time.
+      for(int q = tid; 4 * q < loaded; q += 3 * nt) {
+        int x[3][4] = { { 0, 0, 0, 0 }, { 0, 0, 0, 0 }, { 0, 0, 0, 0 } };
+        PRAGMA_UNROLL
+        for(int r = 0; r < 3; ++r)
+          if(4 * (q + nt * r) < loaded)
+            load_starts(segments, jb + 4 * (q + nt * r), je, x[r]);
+        PRAGMA_UNROLL
+        for(int r = 0; r < 3; ++r)
+          if(4 * (q + nt * r) < loaded) stage(q + nt * r, x[r]);
       }
     }
     if(0 == tid % warp_size) {
