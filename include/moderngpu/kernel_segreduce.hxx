@@ -287,11 +287,14 @@ struct segreduce_tile_f {
     fold_max = 32,
     // Starts (and the start after each) that a thread of an ordinary tile
     // reads ahead into registers; tiles with more than start_regs * nt starts
-    // go to dense_tile().
-#ifndef MGPU_SEGREDUCE_START_REGS
-#define MGPU_SEGREDUCE_START_REGS 2
-#endif
+    // go to dense_tile().  Four for values of up to 4 bytes; wider values
+    // have fewer registers to spare (2^27 doubles in four long segments: 186-
+    // 188 us with three or four against 184-185 us with two).
+#ifdef MGPU_SEGREDUCE_START_REGS
     start_regs = MGPU_SEGREDUCE_START_REGS
+#else
+    start_regs = sizeof(type_t) <= 4 ? 4 : 2
+#endif
   };
   typedef tile_layout_t<W> layout_t;
   typedef cta_segscan_t<nt, type_t> segscan_t;
