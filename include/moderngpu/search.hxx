@@ -316,7 +316,36 @@ struct lbs_partition_search_f {
     int total = count + num_segments;
     int64_t d = (int64_t)spacing * index;
     int diag = (int)(d < total ? d : total);
+    // First j with segments[j] + j >= diag.  The range is cut into quarters
+    // (MGPU_LBS_SEARCH_ARITY parts) a step: the probes of a step are loaded
+    // together, so there are half as many dependent reads as in a binary
+    // search (35,000 splits over 2^24 starts, with the look-back below: 18.7 us
+    // in halves, 17.4-17.9 us in quarters, 20.0 us in eighths, 21.9 us in
+    // sixteenths -- from there on the number of scattered loads counts).
+#ifndef MGPU_LBS_SEARCH_ARITY
+#define MGPU_LBS_SEARCH_ARITY 4
+#endif
+    enum { arity = MGPU_LBS_SEARCH_ARITY };
     int lo = 0, hi = num_segments;
+    while(hi - lo >= arity) {
+      int n = hi - lo;
+      int at[arity - 1], key[arity - 1];
+      PRAGMA_UNROLL
+      for(int q = 0; q < arity - 1; ++q) {
+        at[q] = lo + (int)(((int64_t)n * (q + 1)) / arity);
+        key[q] = segments[at[q]];
+      }
+      // probes are ascending: the first one that is not below diag bounds
+      // the answer from above, the last one below it from below
+      int new_lo = lo, new_hi = hi;
+      PRAGMA_UNROLL
+      for(int q = arity - 2; q >= 0; --q)
+        if((int64_t)key[q] + at[q] >= diag) new_hi = at[q];
+      PRAGMA_UNROLL
+      for(int q = 0; q < arity - 1; ++q)
+        if((int64_t)key[q] + at[q] < diag) new_lo = at[q] + 1;
+      lo = new_lo; hi = new_hi;
+    }
     while(lo < hi) {
       int mid = (int)(((unsigned)lo + (unsigned)hi) / 2);
       if((int64_t)segments[mid] + mid < diag) lo = mid + 1;
@@ -325,10 +354,24 @@ struct lbs_partition_search_f {
     int b = lo, a = min(max(diag - b, 0), count);
     if constexpr(snap > 0) {
       if(index > 0 && d < total) {
+        // Starts in front of the split that lie behind the snapped item
+        // index: counted eight a step, a step's loads in flight together
+        // (one dependent read per start took the kernel from 18 to 23 us on
+        // 2^24 Zipf-distributed segments, where up to 31 starts lie there).
         int a_snap = a - a % snap;
         int back = 0;
-        while(back < window && b - 1 - back >= 0 &&
-          (int)segments[b - 1 - back] > a_snap) ++back;
+        bool more = true;
+        while(more && back < window && b - 1 - back >= 0) {
+          int top = b - 1 - back;           // nearest start not yet seen
+          int v[8];
+          PRAGMA_UNROLL
+          for(int q = 0; q < 8; ++q) v[q] = segments[max(top - q, 0)];
+          PRAGMA_UNROLL
+          for(int q = 0; q < 8; ++q) {
+            if(more && top - q >= 0 && v[q] > a_snap) ++back;
+            else more = false;
+          }
+        }
         if(back < window) { a = a_snap; b -= back; }
       }
       p[2 * index] = (int_t)a;
@@ -339,9 +382,9 @@ struct lbs_partition_search_f {
 };
 
 // It is also used from 2^24 segments on, whatever the number of splits: the
-// scatter kernel reads every start (2^26 of them: 65 us, 22 M: 17 us), the
-// searches read 26 starts per split, the first dozen of which stay in the L2
-// (21 and 12 us; at 2^24 starts the two take the same time).
+// scatter kernel reads every start (2^26 of them: 65 us, 2^24: 24 us, 22 M:
+// 17 us), the searches read some 40 starts per split, the first levels of
+// which stay in the L2 (14, 17.5 and 12 us).
 #ifndef MGPU_LBS_SEARCH_FROM_SEGMENTS
 #define MGPU_LBS_SEARCH_FROM_SEGMENTS (1 << 24)
 #endif
