@@ -65,6 +65,21 @@ def _workspace(nbytes, device):
     return ws
 
 
+_host_words = {}
+
+
+def _pinned_ints(n):
+    """A few ints of pinned host memory per stream, which kernels write
+    straight into (the way the reference's engines take a total back: a store
+    to pinned memory and a wait on the stream, no copy)."""
+    key = torch.cuda.current_stream().cuda_stream
+    t = _host_words.get(key)
+    if t is None or t.numel() < n:
+        t = torch.zeros(max(n, 8), dtype=torch.int32, pin_memory=True)
+        _host_words[key] = t
+    return t
+
+
 def segreduce_tile_size(dtype_code):
     return lib().mgpu_hip_segreduce_tile_size(dtype_code)
 
@@ -389,11 +404,12 @@ def workcreate(created, segments):
     count, num_segments = created.numel(), segments.numel()
     need = lib().mgpu_hip_workcreate_workspace_bytes(count, num_segments)
     ws = _workspace(need, created.device)
-    sizes = torch.zeros(2, dtype=torch.int32, device=created.device)
+    sizes = _pinned_ints(2)
     _check(lib().mgpu_hip_workcreate_upsweep(
         _ptr(created), count, _ptr(segments), num_segments,
         ctypes.c_void_p(sizes.data_ptr()), _ptr(ws), ws.numel(), _stream()))
-    num_new, new_count = (int(x) for x in sizes.tolist())
+    torch.cuda.current_stream().synchronize()
+    num_new, new_count = int(sizes[0]), int(sizes[1])
     outs = [torch.empty(num_new, dtype=torch.int32, device=created.device)
             for _ in range(4)]
     if num_new:
@@ -429,11 +445,12 @@ def inner_join(a, b):
     na, nb = a.numel(), b.numel()
     need = lib().mgpu_hip_inner_join_workspace_bytes(na, nb)
     ws1 = torch.empty(max(int(need), 256), dtype=torch.uint8, device=a.device)
-    count = torch.zeros(1, dtype=torch.int32, device=a.device)
+    count = _pinned_ints(1)
     _check(lib().mgpu_hip_inner_join_count(
         _ptr(a), na, _ptr(b), nb, ctypes.c_void_p(count.data_ptr()),
         _ptr(ws1), ws1.numel(), _stream()))
-    n = int(count.item())
+    torch.cuda.current_stream().synchronize()
+    n = int(count[0])
     pairs = torch.empty((n, 2), dtype=torch.int32, device=a.device)
     if n:
         need = lib().mgpu_hip_inner_join_pairs_workspace_bytes(na, n)
