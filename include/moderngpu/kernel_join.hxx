@@ -2,9 +2,11 @@
 // Returns every pair (i, j) with a[i] equivalent to b[j], ordered by i, then
 // j.  Interface after src/moderngpu/kernel_join.hxx:9-51.  The reference runs
 // two sorted searches (lower and upper bounds of every a key in b); here one
-// search finds the lower bound and the number of matches together.  Then an
-// exclusive scan of the match counts, and a load-balancing search that hands every output pair its
-// a index (the segment) and its position among that key's matches (the rank).
+// search finds the lower bound and the number of matches together, and adds
+// the matches up by tiles of the scan that follows, which so starts from its
+// partials and reads the match counts once.  Then that exclusive scan, and a
+// load-balancing search that hands every output pair its a index (the
+// segment) and its position among that key's matches (the rank).
 #pragma once
 #include "kernel_sortedsearch.hxx"
 #include "kernel_scan.hxx"
@@ -34,6 +36,35 @@ struct join_pairs_f {
   }
 };
 
+// The join's first step with its temporaries in caller-provided device
+// memory: lower[i] = first b key equivalent to a[i], matches[i] = how many
+// are, starts = exclusive scan of matches, *join_count = number of pairs.
+// partitions and samples as for sorted_search_launch; partials holds
+// scan_partials_count(a_count, nv of the scan) ints.
+template<typename search_launch_t, typename a_it, typename b_it,
+  typename comp_t, typename reduction_it>
+void join_count_launch(a_it a, int a_count, b_it b, int b_count, comp_t comp,
+  int* lower, int* matches, int* starts, int* partitions,
+  typename std::iterator_traits<a_it>::value_type* samples, int* partials,
+  reduction_it join_count, context_t& context) {
+  typedef typename scan_launch_default_t<int>::type_t_ scan_launch_t;
+  int scan_nv = scan_launch_t::nv(context);
+  // The search can add up the scan's partials when a tile of its needles
+  // lies in two tiles of the scan at most.
+  bool search_adds = a_count > scan_small_count &&
+    search_launch_t::nv(context) <= scan_nv;
+  if(a_count)
+    sorted_search_launch<bounds_lower, search_launch_t>(a, a_count, b,
+      b_count, lower, comp, partitions, samples, context, matches,
+      search_adds ? partials : nullptr, scan_nv);
+  if(search_adds)
+    scan_finish<scan_type_exc, scan_launch_t>((const int*)matches, a_count,
+      starts, plus_t<int>(), join_count, partials, context);
+  else
+    scan_launch<scan_type_exc, scan_launch_t>((const int*)matches, a_count,
+      starts, plus_t<int>(), join_count, partials, context);
+}
+
 } // namespace detail
 
 template<typename launch_arg_t = empty_t,
@@ -49,28 +80,26 @@ mem_t<int2> inner_join(a_it a, int a_count, b_it b, int b_count,
 
   // Matches of a[i] are b[lower[i] .. lower[i] + matches[i]): one sorted
   // search that finds both bounds of every key from the same tile of b.
+  // starts[i] = where the pairs of a[i] begin in the output; the number of
+  // pairs is read back (the output has to be allocated).
   typedef typename conditional_typedef_t<launch_arg_t,
     detail::sorted_search_launch_default_t>::type_t search_launch_t;
   typedef typename std::iterator_traits<a_it>::value_type type_t;
+  typedef typename detail::scan_launch_default_t<int>::type_t_ scan_launch_t;
+  int nv = search_launch_t::nv(context);
   mem_t<int> lower(a_count, context), matches(a_count, context);
-  if(a_count > 0) {
-    int nv = search_launch_t::nv(context);
-    mem_t<int> partitions(
-      (size_t)div_up((int64_t)a_count + b_count, (int64_t)nv) + 1, context);
-    mem_t<type_t> samples(
-      detail::sorted_search_sample_count(a_count, b_count, nv), context);
-    detail::sorted_search_launch<bounds_lower, search_launch_t>(a, a_count,
-      b, b_count, lower.data(), comp, partitions.data(), samples.data(),
-      context, matches.data());
-  }
-
-  // Where each key's pairs begin in the output, and how many pairs there
-  // are (read back: the output has to be allocated).
   mem_t<int> starts(a_count, context);
+  mem_t<int> partitions(
+    (size_t)div_up((int64_t)a_count + b_count, (int64_t)nv) + 1, context);
+  mem_t<type_t> samples(
+    detail::sorted_search_sample_count(a_count, b_count, nv), context);
+  mem_t<int> partials(detail::scan_partials_count(a_count,
+    scan_launch_t::nv(context)), context);
   mem_t<int> total(1, context);
   const int* lower_data = lower.data();
-  scan<scan_type_exc>(matches.data(), a_count, starts.data(), plus_t<int>(),
-    total.data(), context);
+  detail::join_count_launch<search_launch_t>(a, a_count, b, b_count, comp,
+    lower.data(), matches.data(), starts.data(), partitions.data(),
+    samples.data(), partials.data(), total.data(), context);
   int join_count = from_mem(total)[0];
 
   mem_t<int2> output(join_count, context);

@@ -281,6 +281,15 @@ inline void scan_record(hipEvent_t event, context_t& context) {
   if(hipSuccess != result) throw cuda_exception_t(result);
 }
 
+// What a scan of more than scan_small_count items does once partials[tile]
+// holds the fold of every tile of nv items: the scan of the partials, the
+// total to *reduction, the downsweep.
+template<scan_type_t scan_type, typename launch_t, typename input_it,
+  typename output_it, typename type_t, typename op_t, typename reduction_it>
+void scan_finish(input_it input, int count, output_it output, op_t op,
+  reduction_it reduction, type_t* partials, context_t& context,
+  hipEvent_t event = nullptr);
+
 // The scan with its temporaries in caller-provided device memory:
 // scan_partials_count(count, nv) values of type_t.
 // The event, when not null, is recorded as soon as the reduction has been
@@ -306,7 +315,18 @@ void scan_launch(input_it input, int count, output_it output, op_t op,
   scan_upsweep_f<launch_t, input_it, type_t, op_t>
     up { input, count, op, partials, num_tiles };
   cta_launch<launch_t>(up, xcd_grid(num_tiles), context);
+  scan_finish<scan_type, launch_t>(input, count, output, op, reduction,
+    partials, context, event);
+}
 
+template<scan_type_t scan_type, typename launch_t, typename input_it,
+  typename output_it, typename type_t, typename op_t, typename reduction_it>
+void scan_finish(input_it input, int count, output_it output, op_t op,
+  reduction_it reduction, type_t* partials, context_t& context,
+  hipEvent_t event) {
+
+  int nv = launch_t::nv(context);
+  int num_tiles = div_up(count, nv);
   if(num_tiles <= scan_spine_limit) {
     scan_spine_f<scan_type_exc, scan_spine_nt, spine_vt_t<type_t>::value,
       const type_t*, type_t*, type_t, op_t, reduction_it>

@@ -17,6 +17,7 @@
 #pragma once
 #include "search.hxx"
 #include "cta_load_balance.hxx"
+#include "cta_reduce.hxx"
 #include "launcher.hxx"
 
 BEGIN_MGPU_NAMESPACE
@@ -31,7 +32,12 @@ typedef launch_box_t<arch_gfx950_cta<256, 12, 12> >
 // bound, what a join needs -- from a second search over the same LDS keys.
 // The run of equivalent keys may go on behind the tile's haystack range, so
 // up to `beyond` further keys are staged with it; a needle whose run
-// outlasts those too finishes its search in global memory.
+// outlasts those too finishes its search in global memory.  When totals is
+// not null the counts are also added up by blocks of totals_nv needles
+// (totals[k] += the counts of needles [totals_nv k, totals_nv (k + 1)); the
+// caller has zeroed them), which is what the upsweep of a scan over the
+// counts would compute by reading them again.  totals_nv is at least nv, so
+// a tile's needles lie in two blocks at most.
 template<bounds_t bounds, typename launch_t, typename needles_it,
   typename haystack_it, typename indices_it, typename comp_t,
   bool with_counts = false>
@@ -48,6 +54,8 @@ struct sorted_search_f {
   const int* mp_data;
   int num_tiles;
   int* counts;
+  int* totals;
+  int totals_nv;
 
   MGPU_DEVICE void operator()(int tid, int cta) const {
     typedef typename launch_t::sm_ptx params_t;
@@ -64,6 +72,9 @@ struct sorted_search_f {
     int tile = xcd_tile(cta, num_tiles);
     if(tile >= num_tiles) return;
     __shared__ type_t keys[padded];
+    typedef unsigned long long pair_t;      // two 32-bit sums side by side
+    typedef cta_reduce_t<nt, pair_t> reduce_t;
+    __shared__ typename reduce_t::storage_t reduce_storage;
 
     // tile_range() keeps a tile within nv elements and inside both arrays
     // whatever the splits say.
@@ -106,6 +117,11 @@ struct sorted_search_f {
     // at = byte offset behind the keys known to lie in front of the needle;
     // every round tries to move it on by a power of two.
     int rows = div_up(a_count, (int)nt);
+    // Needles from `second` on belong to the tile's second block of totals.
+    int second = 0;
+    pair_t counted = 0;
+    if constexpr(with_counts)
+      if(totals) second = (range.a_begin / totals_nv + 1) * totals_nv;
     PRAGMA_UNROLL
     for(int i0 = 0; i0 < vt; i0 += lanes) {
       if(i0 >= rows) break;
@@ -166,8 +182,22 @@ struct sorted_search_f {
               }
               upper = lo;
             }
-            counts[range.a_begin + p] = upper - (range.b_begin + lower);
+            int found = upper - (range.b_begin + lower);
+            counts[range.a_begin + p] = found;
+            counted += (pair_t)(unsigned)found <<
+              (range.a_begin + p >= second ? 32 : 0);
           }
+        }
+      }
+    }
+    if constexpr(with_counts) {
+      if(totals) {                  // the same in all threads
+        pair_t sum = reduce_t().reduce(tid, counted, reduce_storage, nt,
+          plus_t<pair_t>(), false);
+        if(!tid) {
+          int block = range.a_begin / totals_nv;
+          if((unsigned)sum) atomicAdd(totals + block, (int)(unsigned)sum);
+          if(sum >> 32) atomicAdd(totals + block + 1, (int)(sum >> 32));
         }
       }
     }
@@ -197,17 +227,27 @@ MGPU_HOST_DEVICE size_t sorted_search_sample_count(int64_t num_needles,
     div_up(num_haystack, (int64_t)search_sample));
 }
 
+// Also clears zero[0 .. zero_count), the totals the search kernel will add
+// its counts to, which saves a launch.
 template<typename needles_it, typename haystack_it, typename type_t>
 struct search_sample_f {
   needles_it needles; haystack_it haystack;
-  int needle_samples;
+  int needle_samples, num_samples;
   type_t* samples;              // needle samples, then haystack samples
+  int* zero; int zero_count;
   MGPU_DEVICE void operator()(int index) const {
     enum { g = search_sample };
-    samples[index] = index < needle_samples ?
-      (type_t)needles[g * index + g - 1] :
-      (type_t)haystack[g * (index - needle_samples)];
+    if(index < zero_count) zero[index] = 0;
+    if(index < num_samples)
+      samples[index] = index < needle_samples ?
+        (type_t)needles[g * index + g - 1] :
+        (type_t)haystack[g * (index - needle_samples)];
   }
+};
+
+struct search_clear_f {
+  int* zero;
+  MGPU_DEVICE void operator()(int index) const { zero[index] = 0; }
 };
 
 template<bounds_t bounds, typename needles_it, typename haystack_it,
@@ -264,14 +304,17 @@ struct sampled_partition_f {
 // num_haystack, nv) + 1 ints, and sorted_search_sample_count() keys (or
 // null: the splits are then found by plain binary searches).
 // counts: null, or (bounds_lower) where the number of haystack keys
-// equivalent to each needle goes.
+// equivalent to each needle goes; totals: null, or div_up(num_needles,
+// totals_nv) ints that receive the sums of the counts by blocks of totals_nv
+// needles (totals_nv >= nv).
 template<bounds_t bounds, typename launch_t, typename needles_it,
   typename haystack_it, typename indices_it, typename comp_t>
 void sorted_search_launch(needles_it needles, int num_needles,
   haystack_it haystack, int num_haystack, indices_it indices, comp_t comp,
   int* mp_data,
   typename std::iterator_traits<needles_it>::value_type* samples,
-  context_t& context, int* counts = nullptr) {
+  context_t& context, int* counts = nullptr, int* totals = nullptr,
+  int totals_nv = 0) {
   typedef typename std::iterator_traits<needles_it>::value_type type_t;
   int64_t total = (int64_t)num_needles + num_haystack;
   if(total >= ((int64_t)1 << 31)) throw cuda_exception_t(hipErrorInvalidValue);
@@ -280,30 +323,38 @@ void sorted_search_launch(needles_it needles, int num_needles,
   int num_tiles = div_up((int)total, nv);
   size_t num_samples = sorted_search_sample_count(num_needles, num_haystack,
     nv);
+  if(totals && (!counts || totals_nv < nv))
+    throw cuda_exception_t(hipErrorInvalidValue);
+  int num_totals = totals ? div_up(num_needles, totals_nv) : 0;
   if(samples && num_samples) {
     int needle_samples = num_needles / search_sample;
     search_sample_f<needles_it, haystack_it, type_t>
-      sample { needles, haystack, needle_samples, samples };
-    transform<256>(sample, num_samples, context);
+      sample { needles, haystack, needle_samples, (int)num_samples, samples,
+        totals, num_totals };
+    transform<256>(sample, std::max(num_samples, (size_t)num_totals),
+      context);
     sampled_partition_f<bounds, needles_it, haystack_it, type_t, comp_t>
       split { needles, haystack, num_needles, num_haystack, nv, comp,
         samples, needle_samples, mp_data };
     transform<256>(split, (size_t)num_tiles + 1, context);
-  } else
+  } else {
+    if(num_totals)
+      transform<256>(search_clear_f { totals }, (size_t)num_totals, context);
     merge_path_partitions_into<bounds>(needles, (int64_t)num_needles,
       haystack, (int64_t)num_haystack, (int64_t)nv, comp, mp_data, context);
+  }
   if constexpr(bounds_lower == bounds) {
     if(counts) {
       sorted_search_f<bounds, launch_t, needles_it, haystack_it, indices_it,
         comp_t, true> k { needles, num_needles, haystack, num_haystack,
-          indices, comp, mp_data, num_tiles, counts };
+          indices, comp, mp_data, num_tiles, counts, totals, totals_nv };
       cta_launch<launch_t>(k, xcd_grid(num_tiles), context);
       return;
     }
   }
   sorted_search_f<bounds, launch_t, needles_it, haystack_it, indices_it,
     comp_t> k { needles, num_needles, haystack, num_haystack, indices, comp,
-      mp_data, num_tiles, nullptr };
+      mp_data, num_tiles, nullptr, nullptr, 0 };
   cta_launch<launch_t>(k, xcd_grid(num_tiles), context);
 }
 

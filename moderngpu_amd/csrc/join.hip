@@ -107,14 +107,10 @@ int mgpu_hip_inner_join_count(const int* a, int a_count, const int* b,
     return (int)hipErrorInvalidValue;
   return guarded(stream, [&](context_t& context) {
     // One search: the lower bound of every a key and the number of b keys
-    // equal to it.
-    if(a_count)
-      detail::sorted_search_launch<bounds_lower, search_launch_t>(a, a_count,
-        b, b_count, ws.lower, less_t<int>(), ws.partitions, ws.samples,
-        context, ws.matches);
-    detail::scan_launch<scan_type_exc, scan_launch_t>(
-      (const int*)ws.matches, a_count, ws.starts, plus_t<int>(), join_count,
-      ws.partials, context);
+    // equal to it; then the scan of those numbers.
+    detail::join_count_launch<search_launch_t>(a, a_count, b, b_count,
+      less_t<int>(), ws.lower, ws.matches, ws.starts, ws.partitions,
+      ws.samples, ws.partials, join_count, context);
   });
 }
 

@@ -46,7 +46,11 @@ def test_sorted_search_disjoint_ranges(oracle, dev):
     (300, 200, 0), (200000, 150000, 1 << 16), (1 << 20, 1 << 20, 1 << 20),
     # runs of equal b keys that go on far behind the tile in which they begin:
     # the match count of an a key is finished outside the tile's own keys
-    (3000, 6000, 3), (20000, 20000, 50), (40, 100000, 1)])
+    (3000, 6000, 3), (20000, 20000, 50), (40, 100000, 1),
+    # just past the size from which the search adds up the scan's partials:
+    # no match at all, a handful of b keys, many a keys against one sample step
+    (16385, 16385, 1 << 30), (16385, 3, 1), (70001, 9, 4),
+    ((1 << 22) + 4097, 1000, 1 << 12)])
 def test_inner_join_matches_oracle(oracle, dev, na, nb, hi):
     import moderngpu_amd as m
     rng = np.random.default_rng(na * 17 + nb)
