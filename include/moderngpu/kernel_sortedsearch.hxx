@@ -216,7 +216,10 @@ struct sorted_search_f {
 // is one, which the diagonals of the tiles are -- and only the last
 // log2(search_sample) steps touch the inputs themselves, within one window of
 // search_sample keys of each.
-enum { search_sample = 1024, search_sample_min_total = 1 << 22 };
+#ifndef MGPU_SEARCH_SAMPLE
+#define MGPU_SEARCH_SAMPLE 1024
+#endif
+enum { search_sample = MGPU_SEARCH_SAMPLE, search_sample_min_total = 1 << 22 };
 
 // Keys of sample storage sorted_search_launch needs (0: no sampling).
 MGPU_HOST_DEVICE size_t sorted_search_sample_count(int64_t num_needles,
