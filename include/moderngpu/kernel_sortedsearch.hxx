@@ -66,12 +66,15 @@ struct sorted_search_f {
       // staged behind it).
       room = nv + beyond,
       padded = (room & (room - 1)) ? (2 << s_log2((int)room)) : room,
-      lanes = 2                     // searches a thread runs side by side
+      lanes = 2,                    // searches a thread runs side by side
+      // keys looked at from the lower bound on for the upper bound, less one;
+      // the LDS array goes on that far behind its padded size
+      window = with_counts ? 8 : 0
     };
     static_assert(beyond <= nt, "one more key per thread at most");
     int tile = xcd_tile(cta, num_tiles);
     if(tile >= num_tiles) return;
-    __shared__ type_t keys[padded];
+    __shared__ type_t keys[padded + window];
     typedef unsigned long long pair_t;      // two 32-bit sums side by side
     typedef cta_reduce_t<nt, pair_t> reduce_t;
     __shared__ typename reduce_t::storage_t reduce_storage;
@@ -105,7 +108,8 @@ struct sorted_search_f {
       type_t filler = haystack[range.b_begin + staged - 1];
       if(with_counts && b_count + tid < staged)
         keys[b_count + tid] = hay_beyond;
-      for(int j = staged + tid; j < padded; j += nt) keys[j] = filler;
+      for(int j = staged + tid; j < padded + window; j += nt)
+        keys[j] = filler;
     }
     PRAGMA_UNROLL
     for(int i = 0; i < vt; ++i)
@@ -143,13 +147,17 @@ struct sorted_search_f {
           if(in_front) at[l] += step * sizeof(type_t);
         }
       }
-      // The same over "keys not behind the needle": the upper bound.
+      // The same over "keys not behind the needle": the upper bound.  Runs
+      // of equivalent keys are mostly short, so the search first looks at
+      // the `window` - 1 keys from the lower bound on (three rounds for a
+      // window of eight); only a needle whose run fills that window searches
+      // all the keys again.
       unsigned up[lanes];
       if constexpr(with_counts) {
         PRAGMA_UNROLL
-        for(int l = 0; l < lanes; ++l) up[l] = 0;
+        for(int l = 0; l < lanes; ++l) up[l] = at[l];
         PRAGMA_UNROLL
-        for(int step = padded / 2; step >= 1; step >>= 1) {
+        for(int step = window / 2; step >= 1; step >>= 1) {
           type_t key[lanes];
           PRAGMA_UNROLL
           for(int l = 0; l < lanes; ++l)
@@ -159,6 +167,27 @@ struct sorted_search_f {
           for(int l = 0; l < lanes; ++l) {
             const type_t& mine = needle[i0 + l < vt ? i0 + l : vt - 1];
             if(!comp(mine, key[l])) up[l] += step * sizeof(type_t);
+          }
+        }
+        bool longer = false;
+        PRAGMA_UNROLL
+        for(int l = 0; l < lanes; ++l)
+          longer |= up[l] - at[l] == (window - 1) * sizeof(type_t);
+        if(longer) {
+          PRAGMA_UNROLL
+          for(int l = 0; l < lanes; ++l) up[l] = 0;
+          PRAGMA_UNROLL
+          for(int step = padded / 2; step >= 1; step >>= 1) {
+                type_t key[lanes];
+            PRAGMA_UNROLL
+            for(int l = 0; l < lanes; ++l)
+              key[l] = *(const type_t*)((const char*)keys + up[l] +
+                (step - 1) * sizeof(type_t));
+            PRAGMA_UNROLL
+            for(int l = 0; l < lanes; ++l) {
+              const type_t& mine = needle[i0 + l < vt ? i0 + l : vt - 1];
+              if(!comp(mine, key[l])) up[l] += step * sizeof(type_t);
+            }
           }
         }
       }
