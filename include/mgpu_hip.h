@@ -316,7 +316,11 @@ MGPU_HIP_API int mgpu_hip_sorted_search(const int* needles, int num_needles,
  * reference runs two searches, and the scan of the counts, :14-31): stores the
  * number of pairs to *join_count (device memory, or host memory the device
  * can write) and leaves what step 2 needs in `workspace`
- * (mgpu_hip_inner_join_workspace_bytes(a_count, b_count) bytes). */
+ * (mgpu_hip_inner_join_workspace_bytes(a_count, b_count) bytes).  The count
+ * (never negative) is stored by the kernel in front of the step's last one:
+ * with *join_count in pinned host memory and set to -1 before the call, the
+ * host may take the count as soon as the word is not negative and enqueue
+ * step 2 while that last kernel still runs. */
 MGPU_HIP_API size_t mgpu_hip_inner_join_workspace_bytes(int a_count,
   int b_count);
 MGPU_HIP_API int mgpu_hip_inner_join_count(const int* a, int a_count,

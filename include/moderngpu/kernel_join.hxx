@@ -40,13 +40,15 @@ struct join_pairs_f {
 // memory: lower[i] = first b key equivalent to a[i], matches[i] = how many
 // are, starts = exclusive scan of matches, *join_count = number of pairs.
 // partitions and samples as for sorted_search_launch; partials holds
-// scan_partials_count(a_count, nv of the scan) ints.
+// scan_partials_count(a_count, nv of the scan) ints.  The event, when not
+// null, is recorded as soon as *join_count has been written, which is before
+// the last kernel of the scan.
 template<typename search_launch_t, typename a_it, typename b_it,
   typename comp_t, typename reduction_it>
 void join_count_launch(a_it a, int a_count, b_it b, int b_count, comp_t comp,
   int* lower, int* matches, int* starts, int* partitions,
   typename std::iterator_traits<a_it>::value_type* samples, int* partials,
-  reduction_it join_count, context_t& context) {
+  reduction_it join_count, context_t& context, hipEvent_t event = nullptr) {
   typedef typename scan_launch_default_t<int>::type_t_ scan_launch_t;
   int scan_nv = scan_launch_t::nv(context);
   // The search can add up the scan's partials when a tile of its needles
@@ -59,10 +61,10 @@ void join_count_launch(a_it a, int a_count, b_it b, int b_count, comp_t comp,
       search_adds ? partials : nullptr, scan_nv);
   if(search_adds)
     scan_finish<scan_type_exc, scan_launch_t>((const int*)matches, a_count,
-      starts, plus_t<int>(), join_count, partials, context);
+      starts, plus_t<int>(), join_count, partials, context, event);
   else
     scan_launch<scan_type_exc, scan_launch_t>((const int*)matches, a_count,
-      starts, plus_t<int>(), join_count, partials, context);
+      starts, plus_t<int>(), join_count, partials, context, event);
 }
 
 } // namespace detail
@@ -80,8 +82,10 @@ mem_t<int2> inner_join(a_it a, int a_count, b_it b, int b_count,
 
   // Matches of a[i] are b[lower[i] .. lower[i] + matches[i]): one sorted
   // search that finds both bounds of every key from the same tile of b.
-  // starts[i] = where the pairs of a[i] begin in the output; the number of
-  // pairs is read back (the output has to be allocated).
+  // starts[i] = where the pairs of a[i] begin in the output.  The number of
+  // pairs goes to pinned host memory (the output has to be allocated) and is
+  // there once the event has passed, while the scan's last kernel still
+  // runs.
   typedef typename conditional_typedef_t<launch_arg_t,
     detail::sorted_search_launch_default_t>::type_t search_launch_t;
   typedef typename std::iterator_traits<a_it>::value_type type_t;
@@ -95,12 +99,14 @@ mem_t<int2> inner_join(a_it a, int a_count, b_it b, int b_count,
     detail::sorted_search_sample_count(a_count, b_count, nv), context);
   mem_t<int> partials(detail::scan_partials_count(a_count,
     scan_launch_t::nv(context)), context);
-  mem_t<int> total(1, context);
+  mem_t<int> total(1, context, memory_space_host);
   const int* lower_data = lower.data();
   detail::join_count_launch<search_launch_t>(a, a_count, b, b_count, comp,
     lower.data(), matches.data(), starts.data(), partitions.data(),
-    samples.data(), partials.data(), total.data(), context);
-  int join_count = from_mem(total)[0];
+    samples.data(), partials.data(), total.data(), context, context.event());
+  hipError_t status = hipEventSynchronize(context.event());
+  if(hipSuccess != status) throw cuda_exception_t(status);
+  int join_count = total.data()[0];
 
   mem_t<int2> output(join_count, context);
   transform_lbs<launch_arg_t>(detail::join_pairs_f { output.data() },

@@ -304,7 +304,7 @@ bool launcher_sorted_search(bool upper, needles_it needles, int num_needles,
 }
 
 // inner_join of int keys ordered by less_t<int>: both steps of the layer,
-// with the count read back in between as the header-only path does.
+// with the count taken back in between as the header-only path does.
 template<typename launch_arg_t, typename a_it, typename b_it, typename comp_t>
 bool launcher_inner_join(a_it a, int a_count, b_it b, int b_count, comp_t,
   context_t& context, mem_t<int2>& output) {
@@ -314,10 +314,21 @@ bool launcher_inner_join(a_it a, int a_count, b_it b, int b_count, comp_t,
     launcher_points_to_t<b_it, int>::value) {
     size_t bytes = mgpu_hip_inner_join_workspace_bytes(a_count, b_count);
     mem_t<char> workspace(bytes, context);
-    mem_t<int> total(1, context);
+    // The count goes to a word of pinned host memory, which holds it as soon
+    // as the kernel that stores it has ended: the host looks at the word for
+    // a while (the kernels behind that one may still run) before it falls
+    // back on waiting for the whole stream.
+    mem_t<int> total(1, context, memory_space_host);
+    volatile int* word = total.data();
+    *word = -1;
     launcher_check(mgpu_hip_inner_join_count(a, a_count, b, b_count,
       total.data(), workspace.data(), bytes, context.stream()));
-    int join_count = from_mem(total)[0];
+    for(long spins = 0; *word < 0 && spins < 2000000; ++spins) { }
+    if(*word < 0) {
+      context.synchronize();
+      if(*word < 0) throw cuda_exception_t(hipErrorUnknown);
+    }
+    int join_count = *word;
     output = mem_t<int2>(join_count, context);
     size_t pairs_bytes = mgpu_hip_inner_join_pairs_workspace_bytes(a_count,
       join_count);

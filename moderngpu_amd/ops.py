@@ -7,6 +7,7 @@ Every call goes through the C ABI of libmgpu_hip.so and is enqueued on torch's
 current stream; nothing here computes on the CPU.
 """
 import ctypes
+import time
 
 import torch
 
@@ -78,6 +79,23 @@ def _pinned_ints(n):
         t = torch.zeros(max(n, 8), dtype=torch.int32, pin_memory=True)
         _host_words[key] = t
     return t
+
+
+def _await_word(word, spin_seconds=5e-3):
+    """The value a kernel stores into word[0] (pinned host memory, set to -1
+    before the launch; the kernels store nothing negative).  The store is
+    visible once its kernel has ended, which may be well before the kernels
+    behind it on the stream have: the host looks at the word for a while
+    before it falls back on waiting for the whole stream."""
+    deadline = time.perf_counter() + spin_seconds
+    while word[0] < 0:
+        if time.perf_counter() > deadline:
+            torch.cuda.current_stream().synchronize()
+            break
+    value = int(word[0])
+    if value < 0:
+        raise MgpuError(1)
+    return value
 
 
 def segreduce_tile_size(dtype_code):
@@ -446,11 +464,12 @@ def inner_join(a, b):
     need = lib().mgpu_hip_inner_join_workspace_bytes(na, nb)
     ws1 = torch.empty(max(int(need), 256), dtype=torch.uint8, device=a.device)
     count = _pinned_ints(1)
+    word = count.numpy()
+    word[0] = -1
     _check(lib().mgpu_hip_inner_join_count(
         _ptr(a), na, _ptr(b), nb, ctypes.c_void_p(count.data_ptr()),
         _ptr(ws1), ws1.numel(), _stream()))
-    torch.cuda.current_stream().synchronize()
-    n = int(count[0])
+    n = _await_word(word)
     pairs = torch.empty((n, 2), dtype=torch.int32, device=a.device)
     if n:
         need = lib().mgpu_hip_inner_join_pairs_workspace_bytes(na, n)
