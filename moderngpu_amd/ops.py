@@ -81,21 +81,21 @@ def _pinned_ints(n):
     return t
 
 
-def _await_word(word, spin_seconds=5e-3):
-    """The value a kernel stores into word[0] (pinned host memory, set to -1
-    before the launch; the kernels store nothing negative).  The store is
+def _await_words(words, n, spin_seconds=5e-3):
+    """The values kernels store into words[:n] (pinned host memory, set to -1
+    before the launch; the kernels store nothing negative).  A store is
     visible once its kernel has ended, which may be well before the kernels
-    behind it on the stream have: the host looks at the word for a while
+    behind it on the stream have: the host looks at the words for a while
     before it falls back on waiting for the whole stream."""
     deadline = time.perf_counter() + spin_seconds
-    while word[0] < 0:
+    while min(words[:n]) < 0:
         if time.perf_counter() > deadline:
             torch.cuda.current_stream().synchronize()
             break
-    value = int(word[0])
-    if value < 0:
+    values = [int(w) for w in words[:n]]
+    if min(values) < 0:
         raise MgpuError(1)
-    return value
+    return values
 
 
 def segreduce_tile_size(dtype_code):
@@ -423,11 +423,12 @@ def workcreate(created, segments):
     need = lib().mgpu_hip_workcreate_workspace_bytes(count, num_segments)
     ws = _workspace(need, created.device)
     sizes = _pinned_ints(2)
+    words = sizes.numpy()
+    words[:2] = -1
     _check(lib().mgpu_hip_workcreate_upsweep(
         _ptr(created), count, _ptr(segments), num_segments,
         ctypes.c_void_p(sizes.data_ptr()), _ptr(ws), ws.numel(), _stream()))
-    torch.cuda.current_stream().synchronize()
-    num_new, new_count = int(sizes[0]), int(sizes[1])
+    num_new, new_count = _await_words(words, 2)
     outs = [torch.empty(num_new, dtype=torch.int32, device=created.device)
             for _ in range(4)]
     if num_new:
@@ -465,11 +466,11 @@ def inner_join(a, b):
     ws1 = torch.empty(max(int(need), 256), dtype=torch.uint8, device=a.device)
     count = _pinned_ints(1)
     word = count.numpy()
-    word[0] = -1
+    word[:1] = -1
     _check(lib().mgpu_hip_inner_join_count(
         _ptr(a), na, _ptr(b), nb, ctypes.c_void_p(count.data_ptr()),
         _ptr(ws1), ws1.numel(), _stream()))
-    n = _await_word(word)
+    n, = _await_words(word, 1)
     pairs = torch.empty((n, 2), dtype=torch.int32, device=a.device)
     if n:
         need = lib().mgpu_hip_inner_join_pairs_workspace_bytes(na, n)
