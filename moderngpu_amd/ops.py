@@ -428,14 +428,18 @@ def workcreate(created, segments):
     _check(lib().mgpu_hip_workcreate_upsweep(
         _ptr(created), count, _ptr(segments), num_segments,
         ctypes.c_void_p(sizes.data_ptr()), _ptr(ws), ws.numel(), _stream()))
+    # What the second step takes besides the outputs is put together while the
+    # first one runs.
+    downsweep = lib().mgpu_hip_workcreate_downsweep
+    front = (_ptr(created), count, _ptr(segments), num_segments)
+    back = (_ptr(ws), ws.numel(), _stream())
     num_new, new_count = _await_words(words, 2)
-    outs = [torch.empty(num_new, dtype=torch.int32, device=created.device)
-            for _ in range(4)]
+    # One allocation for the four outputs, each row on a 256-byte boundary.
+    outs = torch.empty((4, (num_new + 63) // 64 * 64), dtype=torch.int32,
+                       device=created.device)[:, :num_new].unbind(0)
     if num_new:
-        _check(lib().mgpu_hip_workcreate_downsweep(
-            _ptr(created), count, _ptr(segments), num_segments,
-            _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]), _ptr(outs[3]),
-            _ptr(ws), ws.numel(), _stream()))
+        _check(downsweep(*front, _ptr(outs[0]), _ptr(outs[1]), _ptr(outs[2]),
+                         _ptr(outs[3]), *back))
     return (new_count,) + tuple(outs)
 
 
