@@ -81,6 +81,28 @@ def test_segreduce_lbs_scan_fuzz(oracle, dev, seed):
             assert np.array_equal(g.cpu().numpy(), x), ("workcreate",) + tag
 
 
+@pytest.mark.parametrize("seed", range(16))
+def test_join_fuzz_many_keys(oracle, dev, seed):
+    """inner_join past the size from which the search kernel adds up the
+    partials of the scan behind it, with runs of equal keys from none to far
+    longer than the window in which the upper bound is looked for first."""
+    import moderngpu_amd as m
+    rng = np.random.default_rng(777000 + seed)
+    for _ in range(4):
+        n = int(rng.choice([16384, 16385, 20000, 50000, 131072, 300001])) + int(rng.integers(0, 5000))
+        h = int(rng.choice([1, 7, 3000, 16385, 50000, 131072, 300001])) + int(rng.integers(0, 5000))
+        run = float(rng.choice([0.01, 0.5, 1, 3, 6, 7, 8, 12, 40, 500]))
+        hi = max(0, int(h / run))
+        if n * run > 3e6:
+            n = int(3e6 / run)
+        a = np.sort(rng.integers(0, hi + 1, size=n)).astype(np.int32)
+        b = np.sort(rng.integers(0, hi + 1, size=h)).astype(np.int32)
+        got = m.inner_join(torch.from_numpy(a).to(dev), torch.from_numpy(b).to(dev))
+        want = oracle.inner_join(a, b)
+        assert tuple(got.shape) == want.shape, (seed, n, h, hi)
+        assert np.array_equal(got.cpu().numpy(), want), (seed, n, h, hi)
+
+
 @pytest.mark.parametrize("seed", range(20))
 def test_search_and_join_fuzz(oracle, dev, seed):
     import moderngpu_amd as m
