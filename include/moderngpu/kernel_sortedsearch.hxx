@@ -121,11 +121,12 @@ struct sorted_search_f {
     // at = byte offset behind the keys known to lie in front of the needle;
     // every round tries to move it on by a power of two.
     int rows = div_up(a_count, (int)nt);
-    // Needles from `second` on belong to the tile's second block of totals.
+    // The tile's needles from `second` on (counted from the tile's first)
+    // belong to its second block of totals.
     int second = 0;
     pair_t counted = 0;
     if constexpr(with_counts)
-      if(totals) second = (range.a_begin / totals_nv + 1) * totals_nv;
+      if(totals) second = totals_nv - range.a_begin % totals_nv;
     PRAGMA_UNROLL
     for(int i0 = 0; i0 < vt; i0 += lanes) {
       if(i0 >= rows) break;
@@ -214,7 +215,7 @@ struct sorted_search_f {
             int found = upper - (range.b_begin + lower);
             counts[range.a_begin + p] = found;
             counted += (pair_t)(unsigned)found <<
-              (range.a_begin + p >= second ? 32 : 0);
+              (p >= second ? 32 : 0);
           }
         }
       }
