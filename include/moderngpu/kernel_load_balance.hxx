@@ -361,12 +361,14 @@ namespace detail {
 
 // Which of the two tile kernels a call uses.  Without cached values the tiles
 // work from coarse splits (2^28 items in 2^24 segments: 210 against 233 us
-// for the call).  With cached values they keep exact splits: the same decode
-// for them took the same time in the tile kernel, but the partition kernel
-// over exact splits streams all the starts right before the tile kernel and
-// leaves them in the memory-side cache, and without that the tile kernel
-// loses what the cheaper partition saves (interval_expand 257 against 256 us
-// as a call, interval_move 647 against 631 us).
+// for the call).  With cached values they keep exact splits: a tile that
+// works from coarse splits can only ask for its segments' values once it has
+// counted its exact splits, and its 32-bit slots and staged starts leave room
+// for fewer CTAs beside the staged values, so the tile kernel loses more than
+// the cheaper partition saves (interval_expand 275 against 256 us as a call,
+// its tile kernel 255 against 228 us; interval_gather 615 against 557 us,
+// interval_move 662 against 635 us; only inner_join's pair step, one item
+// per segment, gained: 159 against 162 us).
 template<typename pointers_t>
 struct lbs_coarse_splits_t {
   enum { value = 0 == tuple_size<pointers_t>::value };
