@@ -108,6 +108,14 @@ protected:
   size_t _cached_bytes;
   size_t _cache_limit;
 
+  // Small pinned host blocks (the words that totals travel back in) are
+  // kept too: hipHostMalloc and hipHostFree cost far more than the kernels
+  // between them.
+  enum { host_block_max = 1 << 16, host_cache_limit = 1 << 20 };
+  std::multimap<size_t, void*> _free_host_blocks;
+  std::unordered_map<void*, size_t> _live_host_blocks;
+  size_t _cached_host_bytes;
+
   static void check(hipError_t result) {
     if(hipSuccess != result) throw cuda_exception_t(result);
   }
@@ -125,6 +133,7 @@ protected:
     check(hipEventCreate(&_timer[1]));
     check(hipEventCreate(&_event));
     _cached_bytes = 0;
+    _cached_host_bytes = 0;
     // Keep at most 1/8 of device memory parked in the cache.
     _cache_limit = _props.totalGlobalMem / 8;
   }
@@ -158,18 +167,34 @@ public:
 
   // Returns every cached block to the driver (waits for the stream first).
   void release_cache() {
-    if(_free_blocks.empty()) return;
+    if(_free_blocks.empty() && _free_host_blocks.empty()) return;
     (void)hipStreamSynchronize(_stream);
     for(auto& kv : _free_blocks) (void)hipFree(kv.second);
     _free_blocks.clear();
     _cached_bytes = 0;
+    for(auto& kv : _free_host_blocks) (void)hipHostFree(kv.second);
+    _free_host_blocks.clear();
+    _cached_host_bytes = 0;
   }
 
   virtual void* alloc(size_t size, memory_space_t space) {
     void* p = nullptr;
     if(!size) return p;
     if(memory_space_host == space) {
-      check(hipHostMalloc(&p, size, hipHostMallocDefault));
+      if(size > host_block_max) {
+        check(hipHostMalloc(&p, size, hipHostMallocDefault));
+        return p;
+      }
+      size_t host_capacity = (size + 255) & ~(size_t)255;
+      auto found = _free_host_blocks.lower_bound(host_capacity);
+      if(found != _free_host_blocks.end()) {
+        p = found->second;
+        host_capacity = found->first;
+        _cached_host_bytes -= host_capacity;
+        _free_host_blocks.erase(found);
+      } else
+        check(hipHostMalloc(&p, host_capacity, hipHostMallocDefault));
+      _live_host_blocks[p] = host_capacity;
       return p;
     }
     size_t capacity = round_size(size);
@@ -195,7 +220,19 @@ public:
   virtual void free(void* p, memory_space_t space) {
     if(!p) return;
     if(memory_space_host == space) {
-      check(hipHostFree(p));
+      auto host = _live_host_blocks.find(p);
+      if(host == _live_host_blocks.end()) {
+        check(hipHostFree(p));
+        return;
+      }
+      size_t host_capacity = host->second;
+      _live_host_blocks.erase(host);
+      if(_cached_host_bytes + host_capacity > host_cache_limit)
+        check(hipHostFree(p));
+      else {
+        _free_host_blocks.emplace(host_capacity, p);
+        _cached_host_bytes += host_capacity;
+      }
       return;
     }
     auto it = _live_blocks.find(p);

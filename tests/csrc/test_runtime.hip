@@ -159,6 +159,21 @@ static int check_memory(context_t& context) {
   pinned.data()[3] = 42;
   mem_t<int> moved = std::move(pinned);
   CHECK(moved.data()[3] == 42 && pinned.data() == nullptr);
+  // A small pinned block that is released comes back for the next request of
+  // its size (totals travel to the host in such blocks, call after call); a
+  // large one goes back to the driver.
+  {
+    int* first = nullptr;
+    {
+      mem_t<int> word(2, context, memory_space_host);
+      first = word.data();
+      first[0] = 7;
+    }
+    mem_t<int> word(2, context, memory_space_host);
+    CHECK(word.data() == first);
+    mem_t<char> large((size_t)1 << 20, context, memory_space_host);
+    large.data()[(1 << 20) - 1] = 1;
+  }
 
   mem_t<int> sorted = fill_random(0, 1000, 5000, true, context);
   std::vector<int> s = from_mem(sorted);
